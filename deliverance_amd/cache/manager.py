@@ -11,7 +11,8 @@ between requests.  Here a pool of fixed size serves all requests:
   keys, or a window of the last w.  Each group has pages of its own; one page id names the
   same page in every slot of the group.
 * A request's *block table* for a group lists the page of each run of ``page_size``
-  positions; the entry is -1 once a window has passed that run and the page went back.
+  positions; the entry is -1 once a window has passed that run and the page went back
+  (pages that hold positions a windowed group keeps for good, ``keep_first``, never do).
 * ``extend`` reserves pages for a request's next tokens (all groups or nothing);
   ``commit`` makes them part of the request and returns pages that a window has passed;
   ``close`` returns everything.
@@ -34,11 +35,13 @@ class OutOfPages(CacheError):
 
 @dataclass(frozen=True)
 class KVGroupSpec:
-    """Cache slots that share pages.  ``window`` None keeps every key."""
+    """Cache slots that share pages.  ``window`` None keeps every key; with a window, the pages that hold
+    a request's first ``keep_first`` positions are never given back while it lives."""
     slots: Tuple[int, ...]
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)
@@ -211,7 +214,8 @@ class CacheManager:
         for g, pool in enumerate(self.pools):
             first = self._first_live_page(g, r.length)     # the next query sits at r.length
             t = r.tables[g]
-            for j in range(min(first, len(t))):
+            kept = -(-max(0, self.groups[g].keep_first) // self.page_size)   # pages of the first tokens stay
+            for j in range(kept, min(first, len(t))):
                 if t[j] >= 0:
                     self._give(g, [t[j]], rid)
                     released.append((g, t[j]))

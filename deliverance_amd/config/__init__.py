@@ -3,7 +3,8 @@ from .specs import (AttentionSpec, ConfigError, DenseFeedForwardSpec, LayerCall,
 from .gpt2 import Gpt2Config
 from .virudra import VirudraConfig
 from .pedatar import PedatarConfig
+from .pafolorn import PafolornConfig
 from .engine_config import EngineConfig
 
 __all__ = ["AttentionSpec", "ConfigError", "DenseFeedForwardSpec", "LayerCall", "LayerSpec",
-           "ModelConfig", "NormSpec", "PositionSpec", "Gpt2Config", "VirudraConfig", "PedatarConfig", "EngineConfig"]
+           "ModelConfig", "NormSpec", "PositionSpec", "Gpt2Config", "VirudraConfig", "PedatarConfig", "PafolornConfig", "EngineConfig"]

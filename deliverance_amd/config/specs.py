@@ -71,6 +71,16 @@ class QueryTemperatureSpec:
 
 
 @dataclass(frozen=True)
+class QKNormSpec:
+    """Queries and keys pass a root-mean-square norm with a plain gain (eps inside the root) before positions
+    act on them.  ``whole``: one norm over all of a token's query entries and one over all of its key entries,
+    before they are split into heads, with gains of those lengths; else one norm a head with a gain of
+    ``head_dim`` entries that the heads share."""
+    eps: float
+    whole: bool = True
+
+
+@dataclass(frozen=True)
 class AttentionSpec:
     kind: str            # "attention"
     width: int           # model width E
@@ -85,6 +95,9 @@ class AttentionSpec:
     v_head_dim: Optional[int] = None         # per-head size of values; None: head_dim
     distance_bias: Optional[DistanceBiasSpec] = None
     query_temperature: Optional[QueryTemperatureSpec] = None
+    qk_norm: Optional["QKNormSpec"] = None   # queries and keys normalised before any rotation
+    score_softcap: float = 0.0               # positive: score <- cap * tanh(score / cap), after the scale
+    keep_first: int = 0                      # with a window: the first keys of a sequence stay visible for good
 
     @property
     def value_dim(self) -> int:
@@ -138,6 +151,42 @@ class SelectiveScanSpec:
     state: int
     dt_rank: int
     conv_taps: int
+
+
+@dataclass(frozen=True)
+class DeltaRuleSpec:
+    """A gated delta-rule mixer.  Per value head a matrix S (``head_dim`` x ``v_head_dim``, 32-bit) is carried from
+    token to token: S <- g * S (a decay in (0, 1) for every row of S), u = beta * (v - S^T k), S <- S + k u^T,
+    o = S^T q.  q and k (``n_kv_heads`` of them, shared by groups of value heads) and v come from projections
+    followed by a short causal filter of ``conv_taps`` taps a channel and SiLU; q and k are scaled to unit length per
+    head (``unit_eps`` under the root) and q by head_dim^-1/2.  beta = logistic of a projection, one a head.
+    The decay is exp(-exp(A_log) * softplus(a + dt_bias)) with one ``A_log`` a head and a projection a that has one
+    entry a head (``decay == "head"``) or one a head and key channel (``"channel"``); ``decay_rank`` > 0: that
+    projection is two matrices with so many numbers in between.  o is divided by its root mean square per head
+    (``norm_eps``), multiplied by a gain shared by the heads and by ``gate`` ("silu" | "sigmoid") of one more
+    projection (two matrices when ``gate_rank`` > 0), and projected back to the width."""
+    kind: str            # "delta_rule"
+    width: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    conv_taps: int
+    norm_eps: float
+    decay: str = "head"
+    decay_rank: int = 0
+    gate: str = "silu"
+    gate_rank: int = 0
+    unit_eps: float = 1e-6
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Several mixers that read the same input; the result is sum_k scales[k] * branches[k](h).  Every branch keeps
+    a cache slot of its own: branch k of a layer call with slot c uses slot c + k."""
+    kind: str            # "parallel"
+    branches: Tuple[object, ...]
+    scales: Tuple[float, ...]
 
 
 @dataclass(frozen=True)
@@ -203,6 +252,10 @@ class LayerSpec:
     weight_prefix: str = ""
     post_block_norm: Optional[NormSpec] = None
     residual_multiplier: float = 1.0
+    # a learned vector of the model's width that multiplies the mixer's / the feed-forward's result, element by
+    # element, after the norm behind it and before it joins the stream (parameters "mixer_scale", "ff_scale")
+    mixer_scale: bool = False
+    ff_scale: bool = False
 
 
 @dataclass(frozen=True)
@@ -238,7 +291,11 @@ class ModelConfig:
     logit_multiplier: float = 1.0
     # logits <- cap * tanh(logits / cap) when positive
     logit_softcap: float = 0.0
+    # a norm on the embedded tokens before the first layer (parameters "embed_norm")
+    embed_norm: Optional[NormSpec] = None
 
     @property
     def n_cache_slots(self) -> int:
-        return 1 + max((c.cache for c in self.schedule), default=-1)
+        def slots(mixer):
+            return len(mixer.branches) if isinstance(mixer, ParallelMixerSpec) else 1
+        return max((c.cache + slots(self.layers[c.layer].mixer) for c in self.schedule), default=0)

@@ -3,8 +3,11 @@
 // is this attention's true 32-bit path and the reference beside the matrix-core kernels.
 //
 // For the token at position p of its sequence, head h, key j in [lo, p]:
-//   s_j = (q . k_j) * scale * temp(p) + bias[h][min(p - j, n_dist - 1)]
+//   s_j = cap((q . k_j) * scale * temp(p)) + bias[h][min(p - j, n_dist - 1)]
 //   temp(p) = 1 + t_coef * ln(floor((p + 1) / t_every) + 1)          (1 when t_every is 0)
+//   cap(s) = softcap * tanh(s / softcap)                              (s itself when softcap is 0)
+// With a window w the keys are j in [p - w + 1, p] and, with keep_first, also j < keep_first: the first keys of a
+// sequence stay visible at their true positions.
 //   w = softmax(s),  o = sum_j w_j v_j                                 (all in 32-bit)
 // `bias` (optional) is a table by distance, [Hq][n_dist], 32-bit: whoever owns the rule that turns a
 // distance into a learned value (buckets, slopes) writes it out once per layer up to the distance from
@@ -24,7 +27,7 @@ attn_rel_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cac
                     const int* __restrict__ block_table, int max_blocks,
                     const int* __restrict__ seq_of_token, const int* __restrict__ positions,
                     int Hq, int Hkv, int D, int Dv, int page, float scale, int window,
-                    const float* __restrict__ bias, int n_dist, float t_coef, int t_every,
+                    const float* __restrict__ bias, int n_dist, float t_coef, int t_every, float softcap, int keep_first,
                     T* __restrict__ out, int out_ld) {
   __shared__ float qs[REL_MAX_D];
   __shared__ float ps[DA_WAVE];
@@ -49,9 +52,13 @@ attn_rel_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cac
 #pragma unroll
   for (int i = 0; i < REL_MAX_D / DA_WAVE; ++i) acc[i] = 0.f;
 
-  for (int c0 = lo; c0 <= p; c0 += DA_WAVE) {
+  // two runs of keys: the kept first ones that the window has left behind, then the window itself
+  const int kept = keep_first < lo ? keep_first : lo;
+  for (int run = 0; run < 2; ++run) {
+  const int first = run == 0 ? 0 : lo, last = run == 0 ? kept - 1 : p;
+  for (int c0 = first; c0 <= last; c0 += DA_WAVE) {
     const int key = c0 + lane;
-    const bool valid = key <= p && bt[key / page] >= 0;
+    const bool valid = key <= last && bt[key / page] >= 0;
     float s = -INFINITY;
     if (valid) {
       const long long pg = bt[key / page];
@@ -61,6 +68,7 @@ attn_rel_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cac
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot = fmaf(qs[d], to_f32(kr[d]), dot);
       s = dot * qscale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       if (brow) {
         const int dist = p - key;
         s += brow[dist < n_dist ? dist : n_dist - 1];
@@ -73,7 +81,7 @@ attn_rel_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cac
     m = m_new;
     ps[lane] = e;
     __syncthreads();
-    const int cnt = (p - c0 + 1 < DA_WAVE) ? p - c0 + 1 : DA_WAVE;
+    const int cnt = (last - c0 + 1 < DA_WAVE) ? last - c0 + 1 : DA_WAVE;
 #pragma unroll
     for (int i = 0; i < REL_MAX_D / DA_WAVE; ++i) {
       const int d = lane + i * DA_WAVE;
@@ -88,6 +96,7 @@ attn_rel_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cac
     }
     __syncthreads();
   }
+  }
   const float inv = l > 0.f ? 1.0f / l : 0.f;
 #pragma unroll
   for (int i = 0; i < REL_MAX_D / DA_WAVE; ++i) {
@@ -99,7 +108,8 @@ attn_rel_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cac
 extern "C" int da_attn_rel_ref(const void* q, int q_ld, const void* cache, int dtype, const int* block_table,
                                int max_blocks, const int* seq_of_token, const int* positions, int N, int Hq, int Hkv,
                                int D, int Dv, int page, float scale, int window, const float* bias, int n_dist,
-                               float t_coef, int t_every, void* out, int out_ld, void* stream) {
+                               float t_coef, int t_every, float softcap, int keep_first, void* out, int out_ld,
+                               void* stream) {
   DA_REQUIRE(N >= 0 && Hq > 0 && Hkv > 0 && D > 0 && Dv > 0 && page > 0, "attn_rel_ref: bad sizes");
   DA_REQUIRE(Hq % Hkv == 0, "attn_rel_ref: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   DA_REQUIRE(D <= REL_MAX_D && Dv <= REL_MAX_D, "attn_rel_ref: head sizes %d, %d exceed %d", D, Dv, REL_MAX_D);
@@ -107,15 +117,16 @@ extern "C" int da_attn_rel_ref(const void* q, int q_ld, const void* cache, int d
   DA_REQUIRE(window >= 0 && max_blocks > 0, "attn_rel_ref: bad window or block table");
   DA_REQUIRE(!bias || n_dist > 0, "attn_rel_ref: a bias table without entries");
   DA_REQUIRE(t_every >= 0, "attn_rel_ref: bad temperature period %d", t_every);
+  DA_REQUIRE(softcap >= 0.f && keep_first >= 0, "attn_rel_ref: bad score cap or kept first keys");
   if (N == 0) return 0;
   if (dtype == DA_BF16)
     hipLaunchKernelGGL(attn_rel_ref_kernel<bf16_t>, dim3(N * Hq), dim3(DA_WAVE), 0, (hipStream_t)stream,
                        (const bf16_t*)q, q_ld, (const bf16_t*)cache, block_table, max_blocks, seq_of_token, positions,
-                       Hq, Hkv, D, Dv, page, scale, window, bias, n_dist, t_coef, t_every, (bf16_t*)out, out_ld);
+                       Hq, Hkv, D, Dv, page, scale, window, bias, n_dist, t_coef, t_every, softcap, keep_first, (bf16_t*)out, out_ld);
   else
     hipLaunchKernelGGL(attn_rel_ref_kernel<float>, dim3(N * Hq), dim3(DA_WAVE), 0, (hipStream_t)stream,
                        (const float*)q, q_ld, (const float*)cache, block_table, max_blocks, seq_of_token, positions,
-                       Hq, Hkv, D, Dv, page, scale, window, bias, n_dist, t_coef, t_every, (float*)out, out_ld);
+                       Hq, Hkv, D, Dv, page, scale, window, bias, n_dist, t_coef, t_every, softcap, keep_first, (float*)out, out_ld);
   DA_CHECK_LAUNCH("attn_rel_ref");
   return 0;
 }

@@ -1,6 +1,7 @@
 // Small elementwise kernels.
 //   da_gated_act   mid[r, j] = act(gu[r, j]) * gu[r, inner + j]     the two halves of a fused gate | up product
 //   da_softcap     v <- cap * tanh(v / cap)                         in place, 32-bit
+//   da_scale_add_rows  dst[r, c] += mult * scale[c] * src[r, c]     a learned scale per channel, 32-bit
 #include "common.h"
 
 template <typename T, bool FAST>
@@ -37,5 +38,21 @@ extern "C" int da_softcap(float* v, long n, float cap, void* stream) {
   if (n == 0) return 0;
   hipLaunchKernelGGL(softcap_kernel, dim3(da_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, v, n, cap);
   DA_CHECK_LAUNCH("softcap");
+  return 0;
+}
+
+__global__ void scale_add_rows_kernel(const float* __restrict__ src, const float* __restrict__ scale,
+                                      float* __restrict__ dst, long n, int E, float mult) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = fmaf(mult * scale[i % E], src[i], dst[i]);
+}
+
+extern "C" int da_scale_add_rows(const float* src, const float* scale, float* dst, int R, int E, float mult, void* stream) {
+  DA_REQUIRE(R >= 0 && E > 0, "scale_add_rows: bad sizes");
+  if (R == 0) return 0;
+  const long n = (long)R * E;
+  hipLaunchKernelGGL(scale_add_rows_kernel, dim3(da_ceil_div(n, 256)), dim3(256), 0, (hipStream_t)stream, src, scale, dst, n,
+                     E, mult);
+  DA_CHECK_LAUNCH("scale_add_rows");
   return 0;
 }

@@ -32,17 +32,19 @@ class DeviceCache:
             need = needs[slot]
             if isinstance(need, KVNeed):
                 by_shape.setdefault((need.n_kv_heads, need.head_dim, need.window, need.v_head_dim,
-                                     bool(getattr(need, "values_in_keys", False))), []).append(slot)
+                                     bool(getattr(need, "values_in_keys", False)),
+                                     int(getattr(need, "keep_first", 0) or 0)), []).append(slot)
             elif isinstance(need, StateNeed):
                 state_specs.append(StateSpec(slot, need.elems))
                 state_needs[slot] = need
             else:
                 raise TypeError(f"cache slot {slot}: unknown kind of need {need!r}")
-        self.groups: List[KVGroupSpec] = [KVGroupSpec(tuple(slots), h, d, w) for (h, d, w, _, _), slots in by_shape.items()]
+        self.groups: List[KVGroupSpec] = [KVGroupSpec(tuple(slots), h, d, w, keep)
+                                          for (h, d, w, _, _, keep), slots in by_shape.items()]
         # per group: the per-head size of values where it differs from the keys' (None: the same; 0: the values
         # are read out of the key rows and take no room)
         self.v_head_dims: List[Optional[int]] = [0 if shared else (dv if dv != d else None)
-                                                 for (_, d, _, dv, shared) in by_shape]
+                                                 for (_, d, _, dv, shared, _) in by_shape]
         self.n_pages = -(-max_cached_tokens // page_size)
         self.group_of_slot: Dict[int, int] = {}
         self.kv: Dict[int, torch.Tensor] = {}

@@ -97,7 +97,12 @@ _ARGTYPES = {
     "da_attn_prefill_rel": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _VP, _I, _I, _VP],
     "da_rmsnorm": [_VP, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
     "da_rmsnorm_add": [_VP, _VP, _I, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
-    "da_attn_rel_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_rel_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _I, _VP, _VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _I, _VP],
+    "da_delta_rule": [_VP, _I, _I, _I, _I, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I,
+                      _I, _I, _F, _I, _VP],
+    "da_delta_gate_norm": [_VP, _I, _VP, _I, _I, _VP, _I, _F, _I, _VP, _I, _I, _I, _I, _VP],
+    "da_scale_add_rows": [_VP, _VP, _VP, _I, _I, _F, _VP],
     "da_kv_write_split": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_gated_act": [_VP, _I, _I, _VP, _I, _I, _I, _I, _VP],
     "da_softcap": [_VP, ctypes.c_long, _F, _VP],
@@ -328,6 +333,18 @@ def rmsnorm_add(src: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, gain_o
                                      _ptr(next_out), _dt(next_out) if next_out is not None else 0, R, E, _stream()))
 
 
+def scale_add_rows(src: torch.Tensor, scale: torch.Tensor, dst: torch.Tensor, mult: float = 1.0) -> torch.Tensor:
+    """dst[r, c] += mult * scale[c] * src[r, c], all 32-bit: a part's result joins the stream times a learned scale
+    per channel."""
+    _dev(src, scale, dst)
+    _need(src.dtype == dst.dtype == scale.dtype == torch.float32 and src.is_contiguous() and dst.is_contiguous()
+          and scale.is_contiguous() and src.dim() == 2 and src.shape == dst.shape and scale.numel() == src.shape[1],
+          "scale_add_rows: contiguous float32 [R, E], [E] and [R, E] are needed")
+    with _timed("scale_add_rows", 3 * _nbytes(src), 2 * src.numel(), "fp32"):
+        _check(_lib().da_scale_add_rows(_ptr(src), _ptr(scale), _ptr(dst), src.shape[0], src.shape[1], float(mult), _stream()))
+    return dst
+
+
 def gated_act(gu: torch.Tensor, mid: torch.Tensor, act: str) -> torch.Tensor:
     """mid[r, j] = act(gu[r, j]) * gu[r, inner + j]: the halves of a fused gate | up product."""
     _dev(gu, mid)
@@ -542,9 +559,10 @@ def kv_write_split(qkv: torch.Tensor, k_off: int, v_off: int, cache_slot: torch.
 def attention_rel_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
                       positions: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, v_head_dim: int, page: int,
                       scale: float, window: Optional[int], dist_bias: Optional[torch.Tensor], temp_coef: float,
-                      temp_every: int, out: torch.Tensor) -> torch.Tensor:
+                      temp_every: int, out: torch.Tensor, softcap: float = 0.0, keep_first: int = 0) -> torch.Tensor:
     """Plain paged attention with a bias by distance (``dist_bias`` [Hq, n_dist] float32, the last column for every
-    larger distance), a query temperature by position, and values of their own size."""
+    larger distance), a query temperature by position, values of their own size, a cap on the scores
+    (``softcap * tanh(score / softcap)``) and, with a window, ``keep_first`` first keys that stay visible."""
     _dev(q, cache_slot, block_table, seq_of_token, positions, dist_bias, out)
     _rows_2d(q, "q"); _rows_2d(out, "out")
     N = q.shape[0]
@@ -565,7 +583,8 @@ def attention_rel_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: to
     _check(_lib().da_attn_rel_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table), block_table.shape[1],
                                   _ptr(seq_of_token), _ptr(positions), N, n_heads, n_kv_heads, head_dim, v_head_dim, page,
                                   float(scale), int(window or 0), _ptr(dist_bias), n_dist, float(temp_coef),
-                                  int(temp_every), _ptr(out), out.stride(0), _stream()))
+                                  int(temp_every), float(softcap), int(keep_first if window else 0), _ptr(out),
+                                  out.stride(0), _stream()))
     return out
 
 
@@ -981,9 +1000,10 @@ def attention_prefill_rel(q: torch.Tensor, cache_slot: torch.Tensor, block_table
 def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int, n_kv_heads: int,
                         head_dim: int, v_head_dim: int, scale: float, window: Optional[int],
                         dist_bias: Optional[torch.Tensor], temp_coef: float, temp_every: int,
-                        out: torch.Tensor) -> torch.Tensor:
-    """Attention of every row of the step with a bias by distance, a query temperature and values of their own
-    size (each optional).  In bfloat16, with keys and values of one size that is a multiple of 16 up to 128 and a
+                        out: torch.Tensor, softcap: float = 0.0, keep_first: int = 0) -> torch.Tensor:
+    """Attention of every row of the step with a bias by distance, a query temperature, values of their own
+    size, a cap on the scores and first keys that a window keeps (each optional; the last two run on the plain
+    kernel).  In bfloat16, with keys and values of one size that is a multiple of 16 up to 128 and a
     bias row that fits the prefill kernel's LDS copy, the one-token sequences go to the decode kernel and the
     portions to the prefill kernel (their forms with these extras); 32-bit, the reference mode and every other
     shape use the plain kernel for all rows."""
@@ -1007,6 +1027,7 @@ def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: i
                 2 * pairs * n_heads * (D + v_head_dim))
 
     tuned = (_MODE == "tuned" and q.dtype == torch.bfloat16 and v_head_dim == D and D % 16 == 0
+             and softcap == 0.0 and not (window and keep_first)
              and D <= PREFILL_REL_MAX_HEAD_DIM and cache_slot.dim() == 5 and q.stride(0) % 8 == 0
              and q.data_ptr() % 16 == 0 and (dist_bias is None or dist_bias.shape[1] <= PREFILL_REL_MAX_DIST))
     if tuned:
@@ -1025,7 +1046,7 @@ def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: i
         return out
     with _timed("attention_plain", *cost(0, ctx.n_seqs), "fp32" if q.dtype == torch.float32 else "bf16"):
         return attention_rel_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, n_kv_heads, head_dim,
-                                 v_head_dim, page, scale, window, dist_bias, temp_coef, temp_every, out)
+                                 v_head_dim, page, scale, window, dist_bias, temp_coef, temp_every, out, softcap, keep_first)
 
 
 def gated_linear(ctx, h: torch.Tensor, gate_up: torch.Tensor, mid: torch.Tensor, act: str) -> torch.Tensor:
@@ -1387,4 +1408,103 @@ def selective_scan(ctx, x: torch.Tensor, raw_dt: torch.Tensor, bc: torch.Tensor,
                                         _dt(d) if d is not None else 0, _ptr(state), ld, _ptr(ctx.state_slots), _ptr(ctx.q_start),
                                         _ptr(y), y.stride(0), ctx.n_seqs, inner, n_state, chunk, max_chunks, _ptr(cs), _ptr(cd),
                                         _stream()))
+    return y
+
+
+# ------------------------------------------------------------------------------- gated delta rule, attention extras
+DELTA_MAX_DIM = 256          # key entries a head of the delta rule (csrc/delta.hip)
+PREPARE_MAX_ROT = 256        # turned entries a head that ``attn_prepare`` takes (csrc/attn_prepare.hip)
+
+
+def attn_prepare(raw: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, v_head_dim: int,
+                 q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float, whole: bool,
+                 positions: torch.Tensor, speeds: Optional[torch.Tensor], dims: int, interleaved: bool, q_out: torch.Tensor,
+                 cache_slot: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], page: int) -> torch.Tensor:
+    """From the 32-bit rows of a q | k | v product: queries and keys normalised (``whole``: one root mean square
+    over all of a token's query entries and one over all its key entries, gains of those lengths; else head by
+    head with gains of ``head_dim`` entries; no gains: no norm), their first ``dims`` entries turned by the
+    position (``speeds`` float64 [dims / 2]; pairs (2i, 2i + 1) when ``interleaved``, else (i, i + dims / 2)),
+    the queries stored in ``q_out`` and keys and values in their cache rows ``slot_map`` (a page of the slot
+    holds Hkv * page * D keys, then Hkv * Dv * page values)."""
+    _dev(raw, q_gain, k_gain, positions, speeds, q_out, cache_slot, slot_map)
+    _rows_2d(raw, "raw"); _rows_2d(q_out, "q_out")
+    N = raw.shape[0]
+    q_cols, k_cols, v_cols = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_head_dim
+    _need(raw.dtype == torch.float32 and raw.shape[1] >= q_cols + k_cols + v_cols, "attn_prepare: raw must be float32 [N, q | k | v]")
+    _need(q_out.shape[0] == N and q_out.shape[1] >= q_cols, "attn_prepare: q_out must be [N, Hq * D]")
+    _need((q_gain is None) == (k_gain is None), "attn_prepare: a norm needs both gains")
+    if q_gain is not None:
+        nq, nk = (q_cols, k_cols) if whole else (head_dim, head_dim)
+        _need(q_gain.is_contiguous() and k_gain.is_contiguous() and q_gain.numel() == nq and k_gain.numel() == nk,
+              f"attn_prepare: gains of {nq} and {nk} entries are needed")
+    _need(dims % 2 == 0 and 0 <= dims <= min(head_dim, PREPARE_MAX_ROT), f"attn_prepare: {dims} turned entries of {head_dim}")
+    if dims:
+        _need(positions.dtype == torch.int32 and positions.numel() >= N, "attn_prepare: positions must be int32 [N]")
+        _need(speeds is not None and speeds.dtype == torch.float64 and speeds.is_contiguous() and speeds.numel() >= dims // 2,
+              "attn_prepare: speeds must be float64 [dims / 2]")
+    if cache_slot is not None:
+        _need(slot_map is not None and slot_map.dtype == torch.int32 and slot_map.numel() >= N, "attn_prepare: slot_map must be int32 [N]")
+        _need(cache_slot.is_contiguous() and cache_page_elems(cache_slot) == n_kv_heads * page * (head_dim + v_head_dim),
+              "attn_prepare: a page of the cache slot does not hold Hkv * page * (D + Dv) entries")
+        _need(cache_slot.dtype == q_out.dtype, "attn_prepare: cache and queries differ in dtype")
+    with _timed("attn_prepare", N * (q_cols + k_cols + v_cols) * (4 + q_out.element_size()), 8 * N * (q_cols + k_cols), "fp32"):
+        _check(_lib().da_attn_prepare(_ptr(raw), raw.stride(0), n_heads, n_kv_heads, head_dim, v_head_dim, _ptr(q_gain),
+                                      _dt(q_gain) if q_gain is not None else 0, _ptr(k_gain),
+                                      _dt(k_gain) if k_gain is not None else 0, float(eps), int(bool(whole)), _ptr(positions),
+                                      _ptr(speeds) if dims else None, int(dims), int(bool(interleaved)), _ptr(q_out),
+                                      _dt(q_out), q_out.stride(0), _ptr(cache_slot),
+                                      _ptr(slot_map) if cache_slot is not None else None, int(page), N, _stream()))
+    return q_out
+
+
+def delta_rule(ctx, qkv: torch.Tensor, k_off: int, v_off: int, beta_raw: torch.Tensor, decay_raw: torch.Tensor,
+               dt_bias: torch.Tensor, rate: torch.Tensor, state: torch.Tensor, o: torch.Tensor, n_heads: int,
+               n_kv_heads: int, head_dim: int, v_head_dim: int, channel_decay: bool, unit_eps: float,
+               write: bool = True, decay_off: int = 0) -> torch.Tensor:
+    """The gated delta rule over every sequence of the step (see csrc/delta.hip).  ``qkv`` [N, q | k | v] after the
+    filters; ``beta_raw`` [N, H] and ``decay_raw`` [N, H] (or [N, H * D] with ``channel_decay``; from column
+    ``decay_off`` on, so that both may be the rows of one product) are 32-bit sums before their functions; ``rate`` = exp(A_log) [H]; ``state`` [slots, >= H * Dv * D] is read at each portion's
+    start and, with ``write``, written at its end; ``o`` [N, H * Dv] 32-bit."""
+    _dev(qkv, beta_raw, decay_raw, dt_bias, rate, state, o)
+    for t_, nm in ((qkv, "qkv"), (beta_raw, "beta_raw"), (decay_raw, "decay_raw"), (o, "o")):
+        _rows_2d(t_, nm)
+    N = qkv.shape[0]
+    H, G, D, Dv = n_heads, n_kv_heads, head_dim, v_head_dim
+    ld = _state_args(state, "delta_rule")
+    n_decay = H * D if channel_decay else H
+    _need(H % G == 0 and 1 <= D <= DELTA_MAX_DIM, f"delta_rule: {H} heads on {G} key heads of {D} entries")
+    _need(k_off >= G * D and v_off >= k_off + G * D and qkv.shape[1] >= v_off + H * Dv, "delta_rule: q, k and v leave the row")
+    _need(beta_raw.shape[0] == N and decay_raw.shape[0] == N and o.shape[0] == N, "delta_rule: rows differ")
+    _need(beta_raw.dtype == decay_raw.dtype == o.dtype == torch.float32 and beta_raw.shape[1] >= H
+          and decay_raw.shape[1] >= decay_off + n_decay and o.shape[1] >= H * Dv, "delta_rule: beta, decay and o must be float32 of H, H (* D) and H * Dv columns")
+    _need(dt_bias.dtype == rate.dtype == torch.float32 and dt_bias.is_contiguous() and rate.is_contiguous()
+          and dt_bias.numel() == n_decay and rate.numel() == H, "delta_rule: dt_bias and rate must be float32")
+    _need(ld >= H * Dv * D, "delta_rule: the state row is too short")
+    _need(ctx.q_start.numel() >= ctx.n_seqs + 1 and ctx.state_slots.numel() >= ctx.n_seqs, "delta_rule: the step's arrays are too short")
+    nb = N * ((2 * G * D + H * Dv) * qkv.element_size() + (H + n_decay + H * Dv) * 4) + 2 * ctx.n_seqs * H * Dv * D * 4
+    with _timed("delta_rule", nb, 8 * N * H * D * Dv, "fp32"):
+        _check(_lib().da_delta_rule(_ptr(qkv), _dt(qkv), qkv.stride(0), k_off, v_off, _ptr(beta_raw), beta_raw.stride(0),
+                                    _ptr(decay_raw), decay_raw.stride(0), int(decay_off), _ptr(dt_bias), _ptr(rate), _ptr(state), ld,
+                                    _ptr(ctx.state_slots), _ptr(ctx.q_start), _ptr(o), o.stride(0), ctx.n_seqs, H, G, D, Dv,
+                                    int(bool(channel_decay)), float(unit_eps), int(bool(write)), _stream()))
+    return o
+
+
+def delta_gate_norm(o: torch.Tensor, gate: torch.Tensor, gain: torch.Tensor, eps: float, act: str, n_heads: int,
+                    v_head_dim: int, y: torch.Tensor) -> torch.Tensor:
+    """y[n, h, :] = o[n, h, :] / sqrt(mean(o[n, h, :]^2) + eps) * gain * act(gate[n, h, :]); ``act``: "silu" or
+    "sigmoid"; o 32-bit, gate and y in the step's dtype."""
+    _dev(o, gate, gain, y)
+    for t_, nm in ((o, "o"), (gate, "gate"), (y, "y")):
+        _rows_2d(t_, nm)
+    N, cols = o.shape[0], n_heads * v_head_dim
+    _need(o.dtype == torch.float32 and gate.dtype == y.dtype and gate.shape[0] == N and y.shape[0] == N
+          and o.shape[1] >= cols and gate.shape[1] >= cols and y.shape[1] >= cols, "delta_gate_norm: o float32, gate and y of one dtype, [N, H * Dv]")
+    _need(gain.is_contiguous() and gain.numel() == v_head_dim, "delta_gate_norm: the gain has one entry a value channel")
+    if act not in ("silu", "sigmoid"):
+        raise KernelError(f"delta_gate_norm: unknown gate {act!r}")
+    with _timed("delta_gate_norm", N * cols * (4 + 2 * y.element_size()), 8 * N * cols, "fp32"):
+        _check(_lib().da_delta_gate_norm(_ptr(o), o.stride(0), _ptr(gate), _dt(gate), gate.stride(0), _ptr(gain), _dt(gain),
+                                         float(eps), ACTIVATIONS["silu"] if act == "silu" else 0, _ptr(y), y.stride(0), N,
+                                         n_heads, v_head_dim, _stream()))
     return y

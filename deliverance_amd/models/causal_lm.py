@@ -36,6 +36,8 @@ class CausalLM:
                                     for spec, p in zip(config.layers, params["layers"])]
         self.final_norm = None if config.final_norm is None else \
             build_norm(config.final_norm, params["final_norm"], dtype, device)
+        embed_norm = getattr(config, "embed_norm", None)
+        self.embed_norm = None if embed_norm is None else build_norm(embed_norm, params["embed_norm"], dtype, device)
         head = params["head"]["weight"]
         if head is emb["tokens"] and self.token_table.dtype == dtype:
             self.head_weight = self.token_table            # tied: one buffer, two uses
@@ -53,22 +55,27 @@ class CausalLM:
     # ---- what the cache must provide -----------------------------------------------------
     def cache_needs(self) -> Dict[int, object]:
         """cache slot -> KVNeed / StateNeed of the layer call that writes it."""
+        def of(call):
+            """(cache slot, need) of everything the call's mixer keeps: a mixer made of several mixers names a
+            tuple, whose entry k lives in slot ``call.cache + k``."""
+            need = self.blocks[call.layer].mixer.cache_need()
+            many = need if isinstance(need, (tuple, list)) else (need,)
+            return [(call.cache + k, n) for k, n in enumerate(many) if n is not None]
+
         needs: Dict[int, object] = {}
         for call in self.config.schedule:
-            need = self.blocks[call.layer].mixer.cache_need()
-            if need is None:
-                continue
             if call.write:
-                if call.cache in needs:
-                    raise ValueError(f"cache slot {call.cache} is written by two layer calls")
-                needs[call.cache] = need
+                for slot, need in of(call):
+                    if slot in needs:
+                        raise ValueError(f"cache slot {slot} is written by two layer calls")
+                    needs[slot] = need
         for call in self.config.schedule:
-            need = self.blocks[call.layer].mixer.cache_need()
-            if need is not None and not call.write:
-                if call.cache not in needs:
-                    raise ValueError(f"layer {call.layer} reads cache slot {call.cache} that nothing writes")
-                if needs[call.cache] != need:
-                    raise ValueError(f"layer {call.layer} reads cache slot {call.cache} of another shape")
+            if not call.write:
+                for slot, need in of(call):
+                    if slot not in needs:
+                        raise ValueError(f"layer {call.layer} reads cache slot {slot} that nothing writes")
+                    if needs[slot] != need:
+                        raise ValueError(f"layer {call.layer} reads cache slot {slot} of another shape")
         return needs
 
     # ---- one step ----------------------------------------------------------------------------
@@ -82,6 +89,8 @@ class CausalLM:
         x = ctx.buf("residual", N, self.config.width, torch.float32)
         ops.embed(ctx.tokens, ctx.positions, self.token_table, self.embed_position.embed_table(), x,
                   self.config.embed_scale)
+        if self.embed_norm is not None:             # the stream starts as the norm of the embedded tokens, in 32-bit
+            x = self.embed_norm.forward(ctx, x, out_name="residual_normed", out_dtype=torch.float32)
         debug = ctx.debug_hook is not None          # the reference's stages: AbstractModel.java:1100,1107
         if debug:
             ctx.emit(-1, "input", x)

@@ -6,8 +6,11 @@ the output projection (+ bias) added into the residual stream.
 
 Optional extras, each a record of the spec with its constants: values of a per-head size of their own
 (``v_head_dim``), a learned bias by the distance between query and key (``distance_bias``, a table of
-buckets that the mixer writes out once as a table by distance), and a query temperature that grows with
-the position (``query_temperature``).  Positions enter such a mixer through these only.
+buckets that the mixer writes out once as a table by distance), a query temperature that grows with
+the position (``query_temperature``), a root-mean-square norm of queries and keys before the rotation
+(``qk_norm``: over a token's whole projection or head by head), a cap on the scores (``score_softcap``:
+cap * tanh(score / cap)), and first keys of a sequence that a window never leaves behind (``keep_first``:
+position i sees j <= i when i - j < window or j < keep_first).
 Reference: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:226-420
 (projections :266-291, cache write :315-336, scores/softmax/weighted sum :458-532, output
 projection :385-408); the residual add is TransformerBlock.java:176.
@@ -85,19 +88,34 @@ class CausalSelfAttention(Mixer):
         self.temp_coef, self.temp_every = (float(qt.coef), int(qt.every)) if qt is not None else (0.0, 0)
         if qt is not None and self.temp_every <= 0:
             raise ValueError(f"query temperature period {self.temp_every} must be positive")
-        self.extras = self.dist_bias is not None or self.temp_every > 0 or self.v_head_dim != self.head_dim
+        # a cap on the scores, first keys that a window keeps, and the norm of queries and keys
+        self.softcap = float(getattr(spec, "score_softcap", 0.0) or 0.0)
+        self.keep_first = int(getattr(spec, "keep_first", 0) or 0) if self.window else 0
+        if self.softcap < 0.0 or self.keep_first < 0:
+            raise ValueError(f"score cap {self.softcap} and kept first keys {self.keep_first} must not be negative")
+        qn = getattr(spec, "qk_norm", None)
+        self.qk_norm = qn
+        if qn is not None:
+            nq, nk = (self.q_cols, self.kv_cols) if qn.whole else (self.head_dim, self.head_dim)
+            self.q_gain = to_vector(params["q_norm"], dtype, device)
+            self.k_gain = to_vector(params["k_norm"], dtype, device)
+            if self.q_gain.numel() != nq or self.k_gain.numel() != nk:
+                raise ValueError(f"query and key gains have {self.q_gain.numel()} and {self.k_gain.numel()} entries, "
+                                 f"expected {nq} and {nk}")
+        self.extras = (self.dist_bias is not None or self.temp_every > 0 or self.v_head_dim != self.head_dim
+                       or self.softcap > 0.0 or self.keep_first > 0)
         self.position = None
         if spec.position is not None and spec.position.kind != "none":
             self.position = build_position(spec.position, params.get("position", {}), dtype, device)
 
     def cache_need(self):
         return KVNeed(self.n_kv_heads, self.head_dim, self.window,
-                      None if self.v_head_dim == self.head_dim else self.v_head_dim)
+                      None if self.v_head_dim == self.head_dim else self.v_head_dim, keep_first=self.keep_first)
 
     def _epilogue_write(self) -> bool:
         """Whether the q|k|v product may write keys and values to the cache itself (its epilogue assumes
         keys and values of one size)."""
-        return self.position is None and self.v_head_dim == self.head_dim
+        return self.position is None and self.v_head_dim == self.head_dim and self.qk_norm is None
 
     normed_into = True
 
@@ -132,6 +150,20 @@ class CausalSelfAttention(Mixer):
             # the new keys and values go to the cache in the projection's epilogue
             ops.linear(h, self.qkv_weight, self.qkv_bias, qkv, kv_cache=slot, slot_map=ctx.slot_maps[group],
                        q_cols=self.q_cols)
+        elif self.qk_norm is not None:
+            # the norms act on the product's unrounded 32-bit sums; one kernel then normalises queries and keys,
+            # turns them by the position, stores the queries and writes keys and values to the cache
+            raw = ctx.buf("qkv_raw", N, self.qkv_cols, torch.float32)
+            ops.linear(h, self.qkv_weight, self.qkv_bias, raw)
+            rot = self.position if hasattr(self.position, "speeds") else None
+            if self.position is not None and rot is None:
+                raise ValueError("queries and keys with a norm take a rotation or no position encoding")
+            ops.attn_prepare(raw, self.n_heads, self.n_kv_heads, self.head_dim, self.v_head_dim, self.q_gain, self.k_gain,
+                             self.qk_norm.eps, self.qk_norm.whole, ctx.positions,
+                             None if rot is None else rot.speeds, 0 if rot is None else rot.dims,
+                             True if rot is None else rot.interleaved, qkv[:, :self.q_cols],
+                             slot if call.write else None, ctx.slot_maps[group] if call.write else None,
+                             ctx.cache.page_size)
         else:
             ops.linear(h, self.qkv_weight, self.qkv_bias, qkv)
             if self.position is not None:
@@ -151,7 +183,7 @@ class CausalSelfAttention(Mixer):
         if self.extras:
             ops.paged_attention_rel(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.n_kv_heads, self.head_dim,
                                     self.v_head_dim, self.scale, self.window, self.dist_bias, self.temp_coef,
-                                    self.temp_every, o)
+                                    self.temp_every, o, softcap=self.softcap, keep_first=self.keep_first)
         else:
             ops.paged_attention(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.scale, self.window, o)
         if ctx.debug_hook is not None:      # the reference's stage names (CausalSelfAttention.java:299-301,384)

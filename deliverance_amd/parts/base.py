@@ -13,7 +13,8 @@ Interfaces (shapes: N tokens of the step, E model width):
 * ``Mixer.forward(ctx, h, x, call) -> None``: reads h, *adds* its result to x in place
   (32-bit).  ``call`` is the run-order entry (cache slot, write flag).
   ``Mixer.cache_need()`` says what the mixer keeps between steps: a ``KVNeed`` (pages of keys
-  and values), a ``StateNeed`` (fixed-size state in a slot per request) or None.  A mixer with
+  and values), a ``StateNeed`` (fixed-size state in a slot per request), None, or a tuple of these
+  (a mixer made of several: entry k lives in cache slot ``call.cache + k``).  A mixer with
   state finds everything about the step's rows on the device (``ctx.seq_of_token``,
   ``ctx.positions``, ``ctx.q_start``, ``ctx.state_slots``); ``ops.state_gather`` hands every row
   its sequence's state and ``ops.state_scatter`` keeps the state that each portion's last row
@@ -37,12 +38,14 @@ import torch
 class KVNeed:
     """Pages of keys (``head_dim`` a head) and values (``v_head_dim`` a head; None: the keys' size).
     ``values_in_keys``: nothing is kept for the values, they are the first ``v_head_dim`` entries of the key rows
-    (a page is then ``n_kv_heads * page`` rows of ``head_dim`` entries, token by token)."""
+    (a page is then ``n_kv_heads * page`` rows of ``head_dim`` entries, token by token).
+    ``keep_first``: with a window, the first so many positions of a sequence stay readable for good."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
     v_head_dim: Optional[int] = None
     values_in_keys: bool = False
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)

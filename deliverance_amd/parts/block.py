@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import StepContext, build_feed_forward, build_mixer, build_norm
+from .base import StepContext, build_feed_forward, build_mixer, build_norm, to_vector
 
 
 class Block:
@@ -23,9 +23,24 @@ class Block:
         self.post_ff_norm = norm(spec.post_ff_norm, "post_ff_norm")
         self.post_block_norm = norm(getattr(spec, "post_block_norm", None), "post_block_norm")
         self.residual_multiplier = float(getattr(spec, "residual_multiplier", 1.0))
+        # A learned scale per channel on a part's result ("layer scale").  Behind a norm that can take it into its
+        # gain (``Norm.scaled_by``) it costs nothing; else it is applied while the result joins the stream.
+        self.mixer_scale, self.post_mixer_norm = self._scale(spec, params, "mixer_scale", self.post_mixer_norm, dtype, device)
+        self.ff_scale, self.post_ff_norm = self._scale(spec, params, "ff_scale", self.post_ff_norm, dtype, device)
         self.mixer = build_mixer(spec.mixer, params["mixer"], dtype, device)
         self.feed_forward = None if spec.feed_forward is None else \
             build_feed_forward(spec.feed_forward, params["feed_forward"], dtype, device)
+
+    @staticmethod
+    def _scale(spec, params, key, post, dtype, device):
+        """(scale vector still to apply or None, the norm behind the part)."""
+        if not getattr(spec, key, False):
+            return None, post
+        vec = params[key]
+        fold = getattr(post, "scaled_by", None)
+        if fold is not None:
+            return None, fold(vec)
+        return to_vector(vec, torch.float32, device), post
 
     @staticmethod
     def _normed(ctx, x, pre):
@@ -34,7 +49,7 @@ class Block:
         h = ctx.buf("norm", x.shape[0], x.shape[1], ctx.dtype)      # no norm in front: the stream, converted
         return ops.copy_rows(x, h)
 
-    def _part(self, ctx, x, pre, post, run, run_normed, part=None, h_ready=None, next_pre=None):
+    def _part(self, ctx, x, pre, post, run, run_normed, part=None, h_ready=None, next_pre=None, scale=None):
         """One part of the block.  Parts add into the tensor they are given.  Without a norm behind
         the part (and without a multiplier) that tensor is the residual stream; else the part gets
         a buffer of its own (cleared by a fill kernel of the engine's, so that a recorded step
@@ -44,7 +59,7 @@ class Block:
         normalised input of the part that follows (``next_pre`` of the new stream) when the norm behind
         this part could make it in the same pass (``Norm.add_into``), else None."""
         target = x
-        own = post is not None or self.residual_multiplier != 1.0
+        own = post is not None or self.residual_multiplier != 1.0 or scale is not None
         stores = own and getattr(part, "can_store", False)
         if own:
             target = ctx.buf("part_out", x.shape[0], x.shape[1], torch.float32)
@@ -64,11 +79,15 @@ class Block:
         finally:
             ctx.part_accumulate = True
         if own:
-            add_into = None if post is None or self.residual_multiplier != 1.0 else getattr(post, "add_into", None)
+            add_into = None if post is None or self.residual_multiplier != 1.0 or scale is not None else \
+                getattr(post, "add_into", None)
             if add_into is not None:         # norm, addition and the next part's norm in one pass over the rows
                 return add_into(ctx, target, x, next_pre, next_name="norm_ahead")
             out = target if post is None else post.forward(ctx, target, out_name="post_norm", out_dtype=torch.float32)
-            ops.copy_rows(out, x, accumulate=True, scale=self.residual_multiplier)
+            if scale is not None:
+                ops.scale_add_rows(out, scale, x, self.residual_multiplier)
+            else:
+                ops.copy_rows(out, x, accumulate=True, scale=self.residual_multiplier)
         return None
 
     def forward(self, ctx: StepContext, x: torch.Tensor, call) -> None:
@@ -77,7 +96,7 @@ class Block:
                           lambda h, into: self.mixer.forward(ctx, h, into, call),
                           None if fused is None else (lambda norm, into: fused(ctx, norm, x, call) if into is None
                                                       else fused(ctx, norm, x, call, into=into)), part=self.mixer,
-                          next_pre=None if self.feed_forward is None or ctx.debug_hook is not None else self.pre_ff_norm)
+                          scale=self.mixer_scale, next_pre=None if self.feed_forward is None or ctx.debug_hook is not None else self.pre_ff_norm)
         if ctx.debug_hook is not None:
             ctx.emit(call.layer, "post_attention_residual", x)
         if self.feed_forward is not None:
@@ -86,7 +105,7 @@ class Block:
                        lambda h, into: self.feed_forward.forward(ctx, h, into),
                        None if fused is None else (lambda norm, into: fused(ctx, norm, x) if into is None
                                                    else fused(ctx, norm, x, into=into)), part=self.feed_forward,
-                       h_ready=h_ff)
+                       h_ready=h_ff, scale=self.ff_scale)
             if ctx.debug_hook is not None:
                 chosen = getattr(self.feed_forward, "last_choice", None)
                 if chosen is not None:             # a routed feed-forward: the experts of every row, [N, top]

@@ -11,6 +11,7 @@ from .base import FeedForward, StepContext, register_feed_forward, to_matrix, to
 
 class DenseFeedForward(FeedForward):
     graph_safe = True
+    can_store = True          # with ``ctx.part_accumulate`` off the second product stores instead of adding
 
     def __init__(self, spec, params, dtype, device):
         self.width, self.inner, self.activation = spec.width, spec.inner, spec.activation
@@ -41,7 +42,7 @@ class DenseFeedForward(FeedForward):
         N = h.shape[0]
         mid = ctx.buf("ff_mid", N, self.inner, ctx.dtype)
         ops.linear(h, self.fc_weight, self.fc_bias, mid, act=self.activation)
-        ops.linear(mid, self.proj_weight, self.proj_bias, x, accumulate=True)
+        ops.linear(mid, self.proj_weight, self.proj_bias, x, accumulate=ctx.part_accumulate)
 
 
 register_feed_forward("dense", DenseFeedForward)

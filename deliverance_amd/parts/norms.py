@@ -53,6 +53,18 @@ class RmsNorm(Norm):
         out = ctx.buf(out_name, R, self.width, out_dtype or ctx.dtype)
         return ops.rmsnorm(x, self.weight, self.gain_offset, self.eps, out, rows)
 
+    def scaled_by(self, scale: torch.Tensor) -> "RmsNorm":
+        """This norm followed by a multiplication with ``scale``, element by element, as one norm: its gain is
+        (gain_offset + weight) * scale, worked out once in 32-bit."""
+        import copy
+        if scale.numel() != self.width:
+            raise ValueError(f"a scale of {scale.numel()} entries behind a norm of width {self.width}")
+        out = copy.copy(self)
+        out.weight = ((self.weight.to(torch.float32) + self.gain_offset)
+                      * scale.to(device=self.weight.device, dtype=torch.float32).reshape(-1)).contiguous()
+        out.gain_offset = 0.0
+        return out
+
     def rms_params(self):
         """(gain, gain_offset, eps): for kernels that apply this norm to their own rows."""
         return self.weight, self.gain_offset, self.eps
