@@ -18,7 +18,7 @@ its fraction of the roofline; `--no-extra` leaves those two out.  Prints ONE JSO
 vocabulary, feed-forward parameters that a token uses): decode at batch 1, 8 and 64 and the prefill of 2 x 1,024
 tokens for both, at the layer sizes of GPT-2 124M and 355M, one JSON line; with `--profile-stages` also both
 models' kernel tables (stderr).  `--design pedatar` does the same for a third design beside Virudra (the closest
-of the engine's models to it).
+of the engine's models to it), and `--design pafolorn` for a fourth beside Pedatar.
 """
 import argparse
 import json
@@ -225,10 +225,127 @@ def pedatar_step_flops(c, seq_lens_new):
     return fl
 
 
+def pafolorn_config(name, n_positions=1024):
+    """A Pafolorn of GPT-2 ``name``'s sizes: as many layers, a delta rule with a decay per key channel and a parallel
+    mixer in turn.  Delta rule alone: GPT-2's heads with 64 key and 64 value entries each, 4 taps, decay and gate
+    through low ranks of width / 16 and width / 8.  Parallel: attention and a delta rule with half of GPT-2's heads
+    each (64 entries, the first 32 rotated, a window of 512 keys that keeps the first 4, scores capped at 30).
+    Feed-forwards of four times the width, which with the mixers is about what a GPT-2 layer holds."""
+    g = MODELS[name]
+    E, H = g["n_embd"], g["n_head"]
+    alone = {"heads": H, "kv_heads": H, "dim": 64, "vdim": 64, "conv": 4, "a_rank": E // 16, "g_rank": E // 8}
+    left = {"heads": H // 2, "kv_heads": H // 2, "dim": 64, "vdim": 64, "scale": 64 ** -0.5, "softcap": 30.0,
+            "mask": {"size": 512, "keep_first": 4}, "rot": {"base": 10000.0, "dims": 32}}
+    right = {"heads": H // 2, "kv_heads": H // 2, "dim": 64, "vdim": 64, "conv": 4}
+    mlp = {"kind": "dense", "ff": 4 * E}
+    layers = [{"type": "channel_delta", "mixer": alone, "mlp": mlp} if i % 2 == 0 else
+              {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.5, "right_scale": 0.5}, "mlp": mlp}
+              for i in range(g["n_layer"])]
+    return {"architecture": "Pafolorn", "vocab": 50257, "width": E, "norm": {"eps": 1e-5}, "logit_scale": 0.25,
+            "layers": layers, "max_positions": n_positions,
+            # what decode_run and prefill_run read
+            "vocab_size": 50257, "n_positions": n_positions, "n_layer": g["n_layer"], "n_embd": E}
+
+
+def _pafolorn_delta_params(E, m, channel):
+    qk, v = m["kv_heads"] * m["dim"], m["heads"] * m["vdim"]
+    n = E * (2 * qk + v) + m["heads"] * E + v * E
+    if channel:
+        n += m["a_rank"] * (E + m["heads"] * m["dim"]) + m["g_rank"] * (E + v)
+    else:
+        n += m["heads"] * E + v * E
+    return n
+
+
+def _pafolorn_layer_params(c, L):
+    E, m = c["width"], L["mixer"]
+    if L["type"] == "channel_delta":
+        n = _pafolorn_delta_params(E, m, True)
+    else:
+        a = m["left"]
+        n = E * (a["heads"] * a["dim"] + a["kv_heads"] * (a["dim"] + a["vdim"])) + a["heads"] * a["vdim"] * E
+        n += _pafolorn_delta_params(E, m["right"], False)
+    return n + (2 * E * L["mlp"]["ff"] if L["mlp"] else 0)
+
+
+def pafolorn_step_bytes(c, el, batch, ctx_mean):
+    """What a decode step must read: every matrix once, the delta rules' states and filter inputs (read and written,
+    32-bit), and the keys and values that the windows see."""
+    n, extra = c["vocab"] * c["width"], 0
+    for L in c["layers"]:
+        n += _pafolorn_layer_params(c, L)
+        d = L["mixer"] if L["type"] == "channel_delta" else L["mixer"]["right"]
+        chans = 2 * d["kv_heads"] * d["dim"] + d["heads"] * d["vdim"]
+        extra += batch * 2 * 4 * (d["heads"] * d["vdim"] * d["dim"] + (d["conv"] - 1) * chans)
+        if L["type"] == "parallel":
+            a = L["mixer"]["left"]
+            seen = min(ctx_mean, a["mask"]["size"] + a["mask"]["keep_first"])
+            extra += batch * seen * a["kv_heads"] * (a["dim"] + a["vdim"]) * el
+    return n * el + extra
+
+
+def pafolorn_step_flops(c, seq_lens_new):
+    """Matrix-product flops of a step (the parameters a token uses, twice), the attention's two products over the
+    keys that each row sees, and the delta rule's seven operations a state entry and token."""
+    n = sum(seq_lens_new)
+    fl = 2 * len(seq_lens_new) * c["width"] * c["vocab"]
+    for L in c["layers"]:
+        fl += 2 * n * _pafolorn_layer_params(c, L)
+        d = L["mixer"] if L["type"] == "channel_delta" else L["mixer"]["right"]
+        fl += 7 * n * d["heads"] * d["vdim"] * d["dim"]
+        if L["type"] == "parallel":
+            a = L["mixer"]["left"]
+            w, kf = a["mask"]["size"], a["mask"]["keep_first"]
+            pairs = sum(sum(min(i + 1, w + min(kf, max(i + 1 - w, 0))) for i in range(t)) for t in seq_lens_new)
+            fl += 2 * pairs * a["heads"] * (a["dim"] + a["vdim"])
+    return fl
+
+
+def pafolorn_compare(args):
+    """Decode and prefill of Pafolorn beside Pedatar (the closest of the engine's models: a state per request beside
+    attention, root-mean-square norms, short filters) at the layer sizes of GPT-2 124M and 355M; one JSON line."""
+    import numpy as np
+    el, dkey = 2, "bf16"
+    out = {"metric": "decode tok/s at batch 8 of Pafolorn at GPT-2 124M layer sizes (beside Pedatar at the same sizes: see points)",
+           "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": dkey, "steps": args.steps, "warmup": args.warmup,
+           "data": "synthetic (random weights drawn on the GPU, uniform-random token ids)", "points": {}, "points_frac": {}}
+    for size in ("124m", "355m"):
+        for design in ("pedatar", "pafolorn"):
+            rng = np.random.default_rng(0)
+            cfg = pedatar_config(size) if design == "pedatar" else pafolorn_config(size)
+            nbytes = pedatar_step_bytes if design == "pedatar" else pafolorn_step_bytes
+            model = engine_from_gpu_weights(cfg, "bfloat16", 64, kernels=args.kernels)
+            key = f"{design}_{size}"
+            for b in (1, 8, 64):
+                steps = min(args.steps, 128)
+                d, cm = decode_run(model, cfg, rng, b, args.prompt_len, steps, 8)
+                out["points"][f"{key}_decode_b{b}"] = round(b * steps / d, 1)
+                out["points_frac"][f"{key}_decode_b{b}"] = round(nbytes(cfg, el, b, cm) / (d / steps) / 1e9 / HBM_GBS, 4)
+            fl = pedatar_step_flops(cfg, [1024, 1024]) if design == "pedatar" else pafolorn_step_flops(cfg, [1024, 1024])
+            pf = prefill_run(model, cfg, rng, dkey, flops=fl)
+            out["points"][f"{key}_prefill_2048"] = pf["value"]
+            out["points_frac"][f"{key}_prefill_2048"] = pf["frac"]
+            if args.profile_stages:
+                print(f"==== {key}", file=sys.stderr)
+                kernel_table(model, cfg, rng, args.batch, args.prompt_len)
+            del model
+    out["value"] = out["points"]["pafolorn_124m_decode_b8"]
+    out["config"] = {"model": "pafolorn beside pedatar at gpt2-124m and gpt2-355m layer sizes", "global_batch": 8,
+                     "prompt_len": args.prompt_len,
+                     "pafolorn": "a delta rule with a decay per key channel (GPT-2's heads, 64 key and value entries, 4 taps, low "
+                                 "ranks width / 16 and width / 8) and a parallel mixer (attention beside a delta rule, half of "
+                                 "GPT-2's heads each, window 512 keeping the first 4, cap 30, 32 rotated entries) in turn; "
+                                 "feed-forwards of 4 x width", "parallelism": "single-gpu"}
+    print(json.dumps(out))
+    return 0
+
+
 def design_compare(args):
     """Decode and prefill of another design beside its like at equal sizes; one JSON line."""
     if args.design == "pedatar":
         return pedatar_compare(args)
+    if args.design == "pafolorn":
+        return pafolorn_compare(args)
     return virudra_compare(args)
 
 
@@ -435,10 +552,10 @@ def main():
     ap.add_argument("--pool-tokens", type=int, default=None,
                     help="mixed workload: tokens of cache the pool holds (default: every request at full length; fewer force "
                          "requests out of the cache and back, which the line reports as preemptions)")
-    ap.add_argument("--design", default="gpt2", choices=["gpt2", "virudra", "pedatar"],
+    ap.add_argument("--design", default="gpt2", choices=["gpt2", "virudra", "pedatar", "pafolorn"],
                     help="virudra: that design beside GPT-2 at equal sizes (decode at batch 1, 8, 64 and the prefill of 2,048 "
                          "tokens, at 124M and 355M layer sizes) instead of the default workload; pedatar: that design beside "
-                         "Virudra, likewise")
+                         "Virudra, likewise; pafolorn: that design beside Pedatar, likewise")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
                     help="mixed: only the mixed workload, on --model (64 requests with prompts of 16 to 895 tokens arrive at "
                          "once, prompt portions of 512 tokens run beside the decoding of the others, 128 new tokens each)")
@@ -450,7 +567,7 @@ def main():
     import numpy as np
     from deliverance_amd.random_model import random_model
 
-    if args.design in ("virudra", "pedatar"):
+    if args.design in ("virudra", "pedatar", "pafolorn"):
         return design_compare(args)
     cfg = model_config(args.model, args.layers, args.n_positions)
     full_layers = MODELS[args.model]["n_layer"]
