@@ -11,8 +11,8 @@
 // The columns of S do not meet: column j needs k, q, g, beta and v[j] only.  A column is shared out over 16
 // neighbouring lanes, each with RPL consecutive rows in registers; the two sums over rows are taken inside the
 // lane and then over the 16 lanes by DPP additions.  A wavefront holds 4 columns, a workgroup of 4 wavefronts 16;
-// the grid is (sequences x heads x column blocks), each walking its sequence's portion in order, the next token's
-// numbers asked for before this token's arithmetic.  The order of every sum depends on D only, so a token's result
+// the grid is (sequences x heads x column blocks), each walking its sequence's portion in order; the tokens' numbers
+// come through LDS in blocks (see the kernel).  The order of every sum depends on D only, so a token's result
 // does not depend on how the sequence was cut into steps or on its neighbours in the batch.
 //
 // A request's state row holds S as [H][Dv][D] (a column's rows side by side) at its start; a sequence without a
@@ -56,41 +56,34 @@ struct DeltaArgs {
   float unit_eps, q_scale;
 };
 
-// What a lane needs of one token.
+// What a lane needs of one token, as it stands in LDS.
 template <int RPL>
 struct DeltaToken {
-  float k[RPL], q[RPL], a[RPL];       // a: the decay's argument per row (channel) or in a[0] (head)
-  float v, b;
+  float k[RPL], q[RPL], g[RPL];       // unit k, unit q * D^-1/2, the decay a row (channel-wise decays only)
+  float v, b, gh;                     // the column's value, beta, the head's decay
 };
 
-template <typename T, int RPL>
-__device__ __forceinline__ void delta_load(const DeltaArgs& A, int n, int h, int kh, int col, int row0, bool col_ok,
-                                           DeltaToken<RPL>& t) {
-  const T* row = (const T*)A.qkv + (size_t)n * A.ld;
-#pragma unroll
-  for (int r = 0; r < RPL; ++r) {
-    const int d = row0 + r;
-    const int dc = d < A.D ? d : A.D - 1;                      // a valid place; rows past D count as zero below
-    const float m = d < A.D ? 1.f : 0.f;
-    t.q[r] = to_f32(row[kh * A.D + dc]) * m;
-    t.k[r] = to_f32(row[A.k_off + kh * A.D + dc]) * m;
-    t.a[r] = A.channel ? A.araw[(size_t)n * A.a_ld + A.a_off + h * A.D + dc] + A.dt_bias[h * A.D + dc] : 0.f;
-  }
-  if (!A.channel) t.a[0] = A.araw[(size_t)n * A.a_ld + A.a_off + h] + A.dt_bias[h];
-  t.v = to_f32(row[A.v_off + h * A.Dv + (col_ok ? col : 0)]);
-  t.b = A.braw[(size_t)n * A.b_ld + h];
-}
-
+// Tokens come through LDS in blocks of TB: the whole workgroup loads a block (every number once, coalesced), turns
+// the raw numbers into what the recurrence takes (decays, beta, q and k at unit length: all of that is independent
+// of the state and done for the block's tokens side by side), and only then walks the block token by token.  The
+// next block's loads are in flight meanwhile.  What is left on the path from one token's state to the next is a
+// product, a sum over 16 lanes and a multiply-add.
 template <typename T, int RPL, bool FAST>
 __global__ void __launch_bounds__(256)
 delta_rule_kernel(DeltaArgs A) {
+  constexpr int DP = RPL * DELTA_LPC;                        // key rows, padded
+  constexpr int TB = RPL <= 4 ? 32 : (RPL == 8 ? 16 : 8);    // tokens a block
+  constexpr int TS = 3 * DP + 20;                            // floats a token: q | k | g | 16 values | beta | head decay
+  constexpr int PT = (TB * DP + 255) / 256, PV = (TB * DELTA_CPB + 255) / 256;
+  __shared__ __attribute__((aligned(16))) float stage[TB * TS];
   const int blocks_per_head = (A.Dv + DELTA_CPB - 1) / DELTA_CPB;
   const int cb = blockIdx.x % blocks_per_head;
   const int h = (blockIdx.x / blocks_per_head) % A.H;
   const int s = blockIdx.x / (blocks_per_head * A.H);
   const int kh = h / (A.H / A.G);
-  const int sub = threadIdx.x % DELTA_LPC;
-  const int col = cb * DELTA_CPB + threadIdx.x / DELTA_LPC;
+  const int tid = threadIdx.x, lane = tid % DA_WAVE, wave = tid / DA_WAVE;
+  const int sub = tid % DELTA_LPC;
+  const int col = cb * DELTA_CPB + tid / DELTA_LPC;
   const bool col_ok = col < A.Dv;
   const int row0 = sub * RPL;
   const int first = A.q_start[s], last = A.q_start[s + 1];
@@ -102,38 +95,107 @@ delta_rule_kernel(DeltaArgs A) {
 #pragma unroll
   for (int r = 0; r < RPL; ++r) S[r] = (srow && col_ok && row0 + r < A.D) ? srow[row0 + r] : 0.f;
 
-  DeltaToken<RPL> cur, nxt;
-  if (first < last) delta_load<T, RPL>(A, first, h, kh, col, row0, col_ok, cur);
-  for (int n = first; n < last; ++n) {
-    delta_load<T, RPL>(A, n + 1 < last ? n + 1 : n, h, kh, col, row0, col_ok, nxt);     // the next token's numbers, ahead
-    float qq = 0.f, kk = 0.f;
+  // a thread's share of a block, from memory into registers
+  float rq[PT], rk[PT], ra[PT], rv[PV], rb = 0.f, rh = 0.f;
+  auto fetch = [&](int n0) {
+    const int cnt = last - n0 < TB ? last - n0 : TB;
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) { qq = fmaf(cur.q[r], cur.q[r], qq); kk = fmaf(cur.k[r], cur.k[r], kk); }
-    qq = group_sum<DELTA_LPC>(qq);
-    kk = group_sum<DELTA_LPC>(kk);
-    const float qinv = (FAST ? __builtin_amdgcn_rsqf(qq + A.unit_eps) : 1.0f / sqrtf(qq + A.unit_eps)) * A.q_scale;
-    const float kinv = FAST ? __builtin_amdgcn_rsqf(kk + A.unit_eps) : 1.0f / sqrtf(kk + A.unit_eps);
-    const float beta = delta_logistic<FAST>(cur.b);
-    const float g_head = A.channel ? 1.f : delta_exp<FAST>(-rate * delta_softplus<FAST>(cur.a[0]));
-    float dot = 0.f;
+    for (int i = 0; i < PT; ++i) {
+      const int idx = tid + i * 256, tok = idx / DP, d = idx % DP;
+      const bool ok = tok < cnt && d < A.D;
+      const T* row = (const T*)A.qkv + (size_t)(n0 + (ok ? tok : 0)) * A.ld;
+      const int dc = ok ? d : 0;
+      rq[i] = ok ? to_f32(row[kh * A.D + dc]) : 0.f;
+      rk[i] = ok ? to_f32(row[A.k_off + kh * A.D + dc]) : 0.f;
+      ra[i] = (ok && A.channel) ? A.araw[(size_t)(n0 + tok) * A.a_ld + A.a_off + h * A.D + dc] + A.dt_bias[h * A.D + dc] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < PV; ++i) {
+      const int idx = tid + i * 256, tok = idx / DELTA_CPB, c = cb * DELTA_CPB + idx % DELTA_CPB;
+      const bool ok = tok < cnt && c < A.Dv && idx < TB * DELTA_CPB;
+      rv[i] = ok ? to_f32(((const T*)A.qkv)[(size_t)(n0 + tok) * A.ld + A.v_off + h * A.Dv + c]) : 0.f;
+    }
+    if (tid < cnt) {
+      rb = A.braw[(size_t)(n0 + tid) * A.b_ld + h];
+      rh = A.channel ? 0.f : A.araw[(size_t)(n0 + tid) * A.a_ld + A.a_off + h] + A.dt_bias[h];
+    }
+  };
+  // ... and from registers into LDS, the decays and beta worked out on the way
+  auto park = [&]() {
+#pragma unroll
+    for (int i = 0; i < PT; ++i) {
+      const int idx = tid + i * 256, tok = idx / DP, d = idx % DP;
+      if (PT * 256 == TB * DP || idx < TB * DP) {
+        float* at = stage + tok * TS + d;
+        at[0] = rq[i];
+        at[DP] = rk[i];
+        if (A.channel) at[2 * DP] = delta_exp<FAST>(-rate * delta_softplus<FAST>(ra[i]));
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < PV; ++i) {
+      const int idx = tid + i * 256;
+      if (idx < TB * DELTA_CPB) stage[(idx / DELTA_CPB) * TS + 3 * DP + idx % DELTA_CPB] = rv[i];
+    }
+    if (tid < TB) {
+      stage[tid * TS + 3 * DP + DELTA_CPB] = delta_logistic<FAST>(rb);
+      stage[tid * TS + 3 * DP + DELTA_CPB + 1] = A.channel ? 1.f : delta_exp<FAST>(-rate * delta_softplus<FAST>(rh));
+    }
+  };
+  auto take = [&](int tok, DeltaToken<RPL>& t) {
+    const float* at = stage + tok * TS;
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
-      const float g = A.channel ? delta_exp<FAST>(-rate * delta_softplus<FAST>(cur.a[r])) : g_head;
-      cur.k[r] *= kinv;
-      S[r] *= g;
-      dot = fmaf(S[r], cur.k[r], dot);
+      t.q[r] = at[row0 + r];
+      t.k[r] = at[DP + row0 + r];
+      t.g[r] = A.channel ? at[2 * DP + row0 + r] : 0.f;
     }
-    dot = group_sum<DELTA_LPC>(dot);
-    const float u = beta * (cur.v - dot);
-    float out = 0.f;
+    t.v = at[3 * DP + tid / DELTA_LPC];
+    t.b = at[3 * DP + DELTA_CPB];
+    t.gh = at[3 * DP + DELTA_CPB + 1];
+  };
+
+  if (first < last) fetch(first);
+  for (int n0 = first; n0 < last; n0 += TB) {
+    const int cnt = last - n0 < TB ? last - n0 : TB;
+    __syncthreads();                                 // the block before has been walked
+    park();
+    __syncthreads();
+    // q and k to unit length (q also times D^-1/2): wavefront w takes tokens w, w + 4, ...
+    for (int tok = wave; tok < cnt; tok += 256 / DA_WAVE) {
+      float* at = stage + tok * TS;
+      float qq = 0.f, kk = 0.f;
+      for (int d = lane; d < DP; d += DA_WAVE) { qq = fmaf(at[d], at[d], qq); kk = fmaf(at[DP + d], at[DP + d], kk); }
+      qq = wave_sum(qq);
+      kk = wave_sum(kk);
+      const float qinv = (FAST ? __builtin_amdgcn_rsqf(qq + A.unit_eps) : 1.0f / sqrtf(qq + A.unit_eps)) * A.q_scale;
+      const float kinv = FAST ? __builtin_amdgcn_rsqf(kk + A.unit_eps) : 1.0f / sqrtf(kk + A.unit_eps);
+      for (int d = lane; d < DP; d += DA_WAVE) { at[d] *= qinv; at[DP + d] *= kinv; }
+    }
+    __syncthreads();
+    if (n0 + TB < last) fetch(n0 + TB);              // in flight while this block is walked
+    DeltaToken<RPL> cur, nxt;
+    take(0, cur);
+    for (int tok = 0; tok < cnt; ++tok) {
+      take(tok + 1 < TB ? tok + 1 : tok, nxt);       // the next token's numbers, ahead
+      float dot = 0.f;
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) {
-      S[r] = fmaf(cur.k[r], u, S[r]);
-      out = fmaf(S[r], cur.q[r] * qinv, out);
+      for (int r = 0; r < RPL; ++r) {
+        S[r] *= A.channel ? cur.g[r] : cur.gh;
+        dot = fmaf(S[r], cur.k[r], dot);
+      }
+      dot = group_sum<DELTA_LPC>(dot);
+      const float u = cur.b * (cur.v - dot);
+      float out = 0.f;
+#pragma unroll
+      for (int r = 0; r < RPL; ++r) {
+        S[r] = fmaf(cur.k[r], u, S[r]);
+        out = fmaf(S[r], cur.q[r], out);
+      }
+      out = group_sum<DELTA_LPC>(out);
+      if (sub == 0 && col_ok) A.o[(size_t)(n0 + tok) * A.o_ld + h * A.Dv + col] = out;
+      cur = nxt;
     }
-    out = group_sum<DELTA_LPC>(out);
-    if (sub == 0 && col_ok) A.o[(size_t)n * A.o_ld + h * A.Dv + col] = out;
-    cur = nxt;
   }
   if (srow && col_ok && A.write) {
 #pragma unroll

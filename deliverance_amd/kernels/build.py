@@ -32,7 +32,8 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
 # registers and moves every value out and in again.
 EXTRA_FLAGS = {"attn_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
                "attn_prefill_rel.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
-               "attn_latent_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+               "attn_latent_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+               "attn_window.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 _lib = None
 

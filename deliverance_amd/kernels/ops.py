@@ -98,6 +98,8 @@ _ARGTYPES = {
     "da_rmsnorm": [_VP, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
     "da_rmsnorm_add": [_VP, _VP, _I, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
     "da_attn_rel_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _F, _I, _VP, _I, _VP],
+    "da_attn_window": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _VP, _I, _VP],
+    "da_attn_window_takes": [_I, _I, _I],
     "da_attn_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _I, _VP, _VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _I, _VP],
     "da_delta_rule": [_VP, _I, _I, _I, _I, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I,
                       _I, _I, _F, _I, _VP],
@@ -997,16 +999,44 @@ def attention_prefill_rel(q: torch.Tensor, cache_slot: torch.Tensor, block_table
     return out
 
 
+def attention_window(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, q_start: torch.Tensor,
+                     seq_lens: torch.Tensor, seq0: int, n_seqs: int, max_query_len: int, n_heads: int, n_kv_heads: int,
+                     head_dim: int, v_head_dim: int, page: int, scale: float, window: Optional[int], keep_first: int,
+                     softcap: float, out: torch.Tensor) -> torch.Tensor:
+    """Attention of the sequences ``seq0 .. seq0 + n_seqs - 1`` of a step on the matrix cores, in bfloat16, with keys and
+    values of their own sizes, a cap on the scores and, with a window, ``keep_first`` first keys that stay visible."""
+    _dev(q, cache_slot, block_table, q_start, seq_lens, out)
+    _rows_2d(q, "q"); _rows_2d(out, "out")
+    _need(q.dtype == cache_slot.dtype == out.dtype == torch.bfloat16, "attention_window: q, cache and out must be bfloat16")
+    _need(cache_slot.is_contiguous() and cache_page_elems(cache_slot) == n_kv_heads * page * (head_dim + v_head_dim),
+          "attention_window: a page of the cache slot does not hold Hkv * page * (D + Dv) entries")
+    _need(q.shape[1] == n_heads * head_dim and out.shape[1] == n_heads * v_head_dim and out.shape[0] == q.shape[0],
+          "attention_window: q must be [N, Hq*D] and out [N, Hq*Dv]")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
+          and block_table.shape[0] >= seq0 + n_seqs, "attention_window: block_table must be contiguous int32 [S, max_blocks]")
+    _need(q_start.dtype == torch.int32 and q_start.numel() >= seq0 + n_seqs + 1 and seq_lens.dtype == torch.int32
+          and seq_lens.numel() >= seq0 + n_seqs, "attention_window: q_start must be int32 [S+1] and seq_lens int32 [S]")
+    _check(_lib().da_attn_window(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table), block_table.shape[1],
+                                 _ptr(q_start), _ptr(seq_lens), seq0, n_seqs, max_query_len, n_heads, n_kv_heads, head_dim,
+                                 v_head_dim, page, float(scale), int(window or 0), int(keep_first if window else 0),
+                                 float(softcap), _ptr(out), out.stride(0), _stream()))
+    return out
+
+
+def attention_window_takes(head_dim: int, v_head_dim: int, page: int) -> bool:
+    return bool(_lib().da_attn_window_takes(head_dim, v_head_dim, page))
+
+
 def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int, n_kv_heads: int,
                         head_dim: int, v_head_dim: int, scale: float, window: Optional[int],
                         dist_bias: Optional[torch.Tensor], temp_coef: float, temp_every: int,
                         out: torch.Tensor, softcap: float = 0.0, keep_first: int = 0) -> torch.Tensor:
     """Attention of every row of the step with a bias by distance, a query temperature, values of their own
-    size, a cap on the scores and first keys that a window keeps (each optional; the last two run on the plain
-    kernel).  In bfloat16, with keys and values of one size that is a multiple of 16 up to 128 and a
+    size, a cap on the scores and first keys that a window keeps (each optional).  In bfloat16, with keys and values of one size that is a multiple of 16 up to 128 and a
     bias row that fits the prefill kernel's LDS copy, the one-token sequences go to the decode kernel and the
-    portions to the prefill kernel (their forms with these extras); 32-bit, the reference mode and every other
-    shape use the plain kernel for all rows."""
+    portions to the prefill kernel (their forms with these extras); a cap, kept first keys and values of another size
+    go to the matrix-core kernel for those (head sizes up to 128, no bias table, no temperature); 32-bit, the reference
+    mode and every other shape use the plain kernel for all rows."""
     bt = ctx.block_tables[group]
     page = cache_slot.shape[3] if cache_slot.dim() == 5 else ctx.cache.page_size
     D, nd = head_dim, ctx.n_decode
@@ -1017,12 +1047,16 @@ def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: i
         if not KernelProfiler.enabled or not lens:
             return 0, 0
         keys = pairs = rows = 0
+        span = (window + keep_first) if window else 0
         for s_ in range(first, last):
             t = starts[s_ + 1] - starts[s_]
             n = lens[s_]
-            keys += n
+            keys += min(n, span + t) if span else n
             rows += t
-            pairs += sum(n - t + i + 1 for i in range(t)) if t > 1 else n
+            if span:
+                pairs += sum(min(n - t + i + 1, span) for i in range(t))
+            else:
+                pairs += sum(n - t + i + 1 for i in range(t)) if t > 1 else n
         return (keys * n_kv_heads * (D + v_head_dim) * el + rows * n_heads * (D + v_head_dim) * el,
                 2 * pairs * n_heads * (D + v_head_dim))
 
@@ -1043,6 +1077,18 @@ def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: i
             with _timed("attention_prefill", *cost(nd, ctx.n_seqs)):
                 attention_prefill_rel(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, nd, ctx.n_seqs - nd,
                                       ctx.max_query_len, n_heads, scale, window, dist_bias, temp_coef, temp_every, out)
+        return out
+    if (_MODE == "tuned" and q.dtype == torch.bfloat16 and dist_bias is None and temp_every == 0
+            and attention_window_takes(D, v_head_dim, page) and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0):
+        # decode rows (four key phases a row) and portions (row blocks by the longest portion) in a launch each
+        if nd:
+            with _timed("attention_window_decode", *cost(0, nd)):
+                attention_window(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, 0, nd, 1, n_heads, n_kv_heads, D,
+                                 v_head_dim, page, scale, window, keep_first, softcap, out)
+        if ctx.n_seqs > nd:
+            with _timed("attention_window", *cost(nd, ctx.n_seqs)):
+                attention_window(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, nd, ctx.n_seqs - nd, ctx.max_query_len,
+                                 n_heads, n_kv_heads, D, v_head_dim, page, scale, window, keep_first, softcap, out)
         return out
     with _timed("attention_plain", *cost(0, ctx.n_seqs), "fp32" if q.dtype == torch.float32 else "bf16"):
         return attention_rel_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, n_kv_heads, head_dim,

@@ -403,6 +403,73 @@ def test_attention_sees_one_key_at_every_edge(dtype, tail, case):
     assert r.done == [T]
 
 
+WINDOW_KERNEL_SIZES = [quick(4, 2, 64, 64, 100, 4, 30.0), (2, 1, 128, 128, 300, 70, 0.0), (3, 3, 48, 24, 0, 0, 20.0),
+                       (2, 2, 8, 100, 33, 1, 0.0), (8, 2, 32, 64, 64, 64, 10.0), (2, 1, 40, 72, 7, 0, 3.0)]
+
+
+@pytest.mark.parametrize("page", [16, quick(64)])
+@pytest.mark.parametrize("H,G,D,Dv,window,keep,cap", WINDOW_KERNEL_SIZES)
+def test_window_attention_kernel_against_sums_written_out(H, G, D, Dv, window, keep, cap, page):
+    """The matrix-core kernel alone: single rows behind long pasts and portions of 2 to 300 rows (one, two and four row
+    blocks a workgroup, the last one part-filled) behind pasts of 0 to 500 keys; pages handed out in a shuffled order;
+    pages that neither a window nor the kept first keys reach are gone from the table and hold NaN."""
+    from deliverance_amd.kernels import ops
+    rng = np.random.default_rng(H * 1000 + D + window)
+    scale = 0.7 / np.sqrt(D)
+    decode = [(1, 0), (1, 37), (1, 500), (1, window + keep if window else 64)]
+    portions = [(2, 0), (33, 5), (64, 130), (65, 0), (300, 200), (31, 470)]
+    n_pages = sum(-(-(T + past) // page) for T, past in decode + portions) + 1
+    order = list(rng.permutation(n_pages - 1) + 1)                      # page 0 belongs to nobody and holds NaN
+    elems = G * page * (D + Dv)
+    cache = np.full((n_pages, elems), np.nan)
+    max_blocks = max(-(-(T + past) // page) for T, past in decode + portions) + 2
+    tables, qs, wants = [], [], []
+    for T, past in decode + portions:
+        L = T + past
+        K, V = bf16(rng.normal(size=(L, G, D))), bf16(rng.normal(size=(L, G, Dv)))
+        q = bf16(rng.normal(size=(T, H, D)) * 1.5)
+        lo_all = max(0, past - window + 1) if window else 0             # the first key that any row's window reaches
+        row = np.full(max_blocks, -1, dtype=np.int64)
+        for b in range(-(-L // page)):
+            first, last = b * page, min(L, (b + 1) * page) - 1
+            if last < lo_all and first >= keep:
+                continue                                                # nobody sees this page: it is gone
+            pg = order.pop()
+            row[b] = pg
+            for j in range(first, last + 1):
+                r = j - first
+                for g in range(G):
+                    cache[pg, (g * page + r) * D:(g * page + r + 1) * D] = K[j, g]
+                    cache[pg, G * page * D + g * Dv * page:G * page * D + (g + 1) * Dv * page].reshape(Dv, page)[:, r] = V[j, g]
+        # what was left of a page behind a sequence's end is anything: keep the NaN there
+        tables.append(row)
+        qs.append(q.reshape(T, H * D))
+        o = np.zeros((T, H, Dv))
+        for i in range(T):
+            p_ = past + i
+            js = np.array([j for j in range(p_ + 1) if not window or p_ - j < window or j < keep])
+            for h in range(H):
+                g = h // (H // G)
+                sc = (K[js, g] @ q[i, h]) * scale
+                if cap:
+                    sc = cap * np.tanh(sc / cap)
+                w = np.exp(sc - sc.max())
+                o[i, h] = (w / w.sum()) @ V[js, g]
+        wants.append(o.reshape(T, H * Dv))
+    q_all = dev(np.concatenate(qs), torch.bfloat16)
+    lens = [T + past for T, past in decode + portions]
+    starts = np.concatenate([[0], np.cumsum([T for T, _ in decode + portions])])
+    out = torch.full((q_all.shape[0], H * Dv), float("nan"), dtype=torch.bfloat16, device=DEV)
+    cache_t, bt = dev(cache, torch.bfloat16), dev(np.stack(tables))
+    nd = len(decode)
+    ops.attention_window(q_all, cache_t, bt, dev(starts), dev(lens), 0, nd, 1, H, G, D, Dv, page, scale, window, keep, cap, out)
+    ops.attention_window(q_all, cache_t, bt, dev(starts), dev(lens), nd, len(portions), max(T for T, _ in portions), H, G, D, Dv,
+                         page, scale, window, keep, cap, out)
+    got, want = host(out), np.concatenate(wants)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max()
+
+
 # ------------------------------------------------------------------------------------------ parallel mixers, layer scale
 @pytest.mark.parametrize("dtype", ["float32", quick("bfloat16")])
 def test_parallel_mixers_add_with_their_constants(dtype):

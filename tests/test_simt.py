@@ -40,6 +40,11 @@ RUNS = {
                 "rotation or filter or router_takes or (squared_ramp and bfloat16) or (routed_feed_forward and bfloat16 and not 300) "
                 "or (selective_scan and bfloat16) or (far_key and 31 and bfloat16) or (latent_attention_part and bfloat16 and m0) "
                 "or (whole_prompts and (P or R) and bfloat16) or (mixed_batches and R and bfloat16)"],
+    # a fourth design's kernels and parts (the gated delta rule, its read-out norm, the norm and turn of queries and
+    # keys, attention over a window with kept first keys on its plain and matrix-core forms, parallel mixers) and its
+    # models through the step function
+    "pafolorn": ["tests/test_pafolorn_gpu.py", "-n", "4"] if FULL else
+                ["tests/test_pafolorn_gpu.py", "-n", "3", "-m", QUICK],
     "replay": ["tests/test_replay_gpu.py", "-n", "4"] if FULL else
               ["tests/test_replay_gpu.py", "-n", "2", "-k", "(mixed and (A or B) and not 32) or want_subset or errors_leave or first_tokens"],
     # inner sizes of 32 in an engine step: qkv and fc of seed 11 (and, in the full run, proj of seed 5)
