@@ -56,26 +56,28 @@ struct DeltaArgs {
   float unit_eps, q_scale;
 };
 
-// What a lane needs of one token, as it stands in LDS.
-template <int RPL>
-struct DeltaToken {
-  float k[RPL], q[RPL], g[RPL];       // unit k, unit q * D^-1/2, the decay a row (channel-wise decays only)
-  float v, b, gh;                     // the column's value, beta, the head's decay
-};
-
-// Tokens come through LDS in blocks of TB: the whole workgroup loads a block (every number once, coalesced), turns
-// the raw numbers into what the recurrence takes (decays, beta, q and k at unit length: all of that is independent
-// of the state and done for the block's tokens side by side), and only then walks the block token by token.  The
-// next block's loads are in flight meanwhile.  What is left on the path from one token's state to the next is a
-// product, a sum over 16 lanes and a multiply-add.
+// Tokens come through LDS in blocks of TB: the whole workgroup loads a block (every number once, coalesced) and
+// turns the raw numbers into what the recurrence takes; the next block's loads are in flight while this one is
+// walked.  The walk itself goes four tokens at a time.  With S the state in front of tokens 1..4, P_ts the product
+// of the decays of tokens s+1..t (row by row; P_tt = 1) and G_t = P_t0 the product of the decays of tokens 1..t:
+//     u_t = beta_t (v_t - S^T (G_t k_t) - sum_{s<t} A_ts u_s)        A_ts = sum_d k_t k_s P_ts
+//     o_t = S^T (G_t q_t) + sum_{s<=t} B_ts u_s                       B_ts = sum_d q_t k_s P_ts
+//     S  <- G_4 S + sum_s (P_4s k_s) u_s^T
+// which is the token-by-token rule written out (no quotient of decays anywhere: only products of numbers in (0, 1]).
+// A, B, G_t k_t, G_t q_t and P_4s k_s do not depend on the state: wavefronts work them out for the block's fours
+// side by side.  What is left on the path from one four's state to the next: eight sums over the rows of a column
+// (independent of each other, so their lane exchanges overlap), ten multiply-adds on a column's four u, and the
+// update.  A portion's last four is filled up with tokens that change nothing (decay 1, beta 0, k = q = 0).
 template <typename T, int RPL, bool FAST>
 __global__ void __launch_bounds__(256)
 delta_rule_kernel(DeltaArgs A) {
   constexpr int DP = RPL * DELTA_LPC;                        // key rows, padded
   constexpr int TB = RPL <= 4 ? 32 : (RPL == 8 ? 16 : 8);    // tokens a block
-  constexpr int TS = 3 * DP + 20;                            // floats a token: q | k | g | 16 values | beta | head decay
+  constexpr int TS = 3 * DP + 20;                            // floats a token: q | k | g | 16 values | beta
+  constexpr int NF = TB / 4, FS = DP + 16;                   // fours a block; floats a four: G_4 | A (6) | B (10)
   constexpr int PT = (TB * DP + 255) / 256, PV = (TB * DELTA_CPB + 255) / 256;
   __shared__ __attribute__((aligned(16))) float stage[TB * TS];
+  __shared__ __attribute__((aligned(16))) float fours[NF * FS];
   const int blocks_per_head = (A.Dv + DELTA_CPB - 1) / DELTA_CPB;
   const int cb = blockIdx.x % blocks_per_head;
   const int h = (blockIdx.x / blocks_per_head) % A.H;
@@ -96,32 +98,37 @@ delta_rule_kernel(DeltaArgs A) {
   for (int r = 0; r < RPL; ++r) S[r] = (srow && col_ok && row0 + r < A.D) ? srow[row0 + r] : 0.f;
 
   // a thread's share of a block, from memory into registers
-  float rq[PT], rk[PT], ra[PT], rv[PV], rb = 0.f, rh = 0.f;
+  float rq[PT], rk[PT], ra[PT], rv[PV], rb = 0.f;
+  // (every load is unconditional, from a place that exists, and what does not count is replaced afterwards: a load
+  // under a condition becomes a branch, and the loads would wait for each other)
   auto fetch = [&](int n0) {
     const int cnt = last - n0 < TB ? last - n0 : TB;
 #pragma unroll
     for (int i = 0; i < PT; ++i) {
       const int idx = tid + i * 256, tok = idx / DP, d = idx % DP;
       const bool ok = tok < cnt && d < A.D;
-      const T* row = (const T*)A.qkv + (size_t)(n0 + (ok ? tok : 0)) * A.ld;
-      const int dc = ok ? d : 0;
-      rq[i] = ok ? to_f32(row[kh * A.D + dc]) : 0.f;
-      rk[i] = ok ? to_f32(row[A.k_off + kh * A.D + dc]) : 0.f;
-      ra[i] = (ok && A.channel) ? A.araw[(size_t)(n0 + tok) * A.a_ld + A.a_off + h * A.D + dc] + A.dt_bias[h * A.D + dc] : 0.f;
+      const int tc = tok < cnt ? tok : cnt - 1, dc = d < A.D ? d : A.D - 1;
+      const T* row = (const T*)A.qkv + (size_t)(n0 + tc) * A.ld;
+      const int ac = A.channel ? h * A.D + dc : h;
+      const float xq = to_f32(row[kh * A.D + dc]), xk = to_f32(row[A.k_off + kh * A.D + dc]);
+      const float xa = A.araw[(size_t)(n0 + tc) * A.a_ld + A.a_off + ac] + A.dt_bias[ac];
+      rq[i] = ok ? xq : 0.f;
+      rk[i] = ok ? xk : 0.f;
+      ra[i] = ok ? xa : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < PV; ++i) {
-      const int idx = tid + i * 256, tok = idx / DELTA_CPB, c = cb * DELTA_CPB + idx % DELTA_CPB;
-      const bool ok = tok < cnt && c < A.Dv && idx < TB * DELTA_CPB;
-      rv[i] = ok ? to_f32(((const T*)A.qkv)[(size_t)(n0 + tok) * A.ld + A.v_off + h * A.Dv + c]) : 0.f;
+      const int idx = (tid + i * 256) % (TB * DELTA_CPB), tok = idx / DELTA_CPB, c = cb * DELTA_CPB + idx % DELTA_CPB;
+      const bool ok = tok < cnt && c < A.Dv;
+      const int tc = tok < cnt ? tok : cnt - 1, cc = c < A.Dv ? c : A.Dv - 1;
+      const float xv = to_f32(((const T*)A.qkv)[(size_t)(n0 + tc) * A.ld + A.v_off + h * A.Dv + cc]);
+      rv[i] = ok ? xv : 0.f;
     }
-    if (tid < cnt) {
-      rb = A.braw[(size_t)(n0 + tid) * A.b_ld + h];
-      rh = A.channel ? 0.f : A.araw[(size_t)(n0 + tid) * A.a_ld + A.a_off + h] + A.dt_bias[h];
-    }
+    rb = A.braw[(size_t)(n0 + (tid < cnt ? tid : cnt - 1)) * A.b_ld + h];
   };
-  // ... and from registers into LDS, the decays and beta worked out on the way
-  auto park = [&]() {
+  // ... and from registers into LDS, the decays and beta worked out on the way; tokens past the block's last and
+  // rows past D change nothing
+  auto park = [&](int cnt) {
 #pragma unroll
     for (int i = 0; i < PT; ++i) {
       const int idx = tid + i * 256, tok = idx / DP, d = idx % DP;
@@ -129,7 +136,7 @@ delta_rule_kernel(DeltaArgs A) {
         float* at = stage + tok * TS + d;
         at[0] = rq[i];
         at[DP] = rk[i];
-        if (A.channel) at[2 * DP] = delta_exp<FAST>(-rate * delta_softplus<FAST>(ra[i]));
+        at[2 * DP] = (tok < cnt && d < A.D) ? delta_exp<FAST>(-rate * delta_softplus<FAST>(ra[i])) : 1.f;
       }
     }
 #pragma unroll
@@ -137,30 +144,16 @@ delta_rule_kernel(DeltaArgs A) {
       const int idx = tid + i * 256;
       if (idx < TB * DELTA_CPB) stage[(idx / DELTA_CPB) * TS + 3 * DP + idx % DELTA_CPB] = rv[i];
     }
-    if (tid < TB) {
-      stage[tid * TS + 3 * DP + DELTA_CPB] = delta_logistic<FAST>(rb);
-      stage[tid * TS + 3 * DP + DELTA_CPB + 1] = A.channel ? 1.f : delta_exp<FAST>(-rate * delta_softplus<FAST>(rh));
-    }
-  };
-  auto take = [&](int tok, DeltaToken<RPL>& t) {
-    const float* at = stage + tok * TS;
-#pragma unroll
-    for (int r = 0; r < RPL; ++r) {
-      t.q[r] = at[row0 + r];
-      t.k[r] = at[DP + row0 + r];
-      t.g[r] = A.channel ? at[2 * DP + row0 + r] : 0.f;
-    }
-    t.v = at[3 * DP + tid / DELTA_LPC];
-    t.b = at[3 * DP + DELTA_CPB];
-    t.gh = at[3 * DP + DELTA_CPB + 1];
+    if (tid < TB) stage[tid * TS + 3 * DP + DELTA_CPB] = tid < cnt ? delta_logistic<FAST>(rb) : 0.f;
   };
 
   if (first < last) fetch(first);
   for (int n0 = first; n0 < last; n0 += TB) {
     const int cnt = last - n0 < TB ? last - n0 : TB;
-    __syncthreads();                                 // the block before has been walked
-    park();
-    __syncthreads();
+    const int n_fours = (cnt + 3) / 4;
+    lds_barrier();                                   // the block before has been walked (its stores may still be on their way)
+    park(cnt);
+    lds_barrier();
     // q and k to unit length (q also times D^-1/2): wavefront w takes tokens w, w + 4, ...
     for (int tok = wave; tok < cnt; tok += 256 / DA_WAVE) {
       float* at = stage + tok * TS;
@@ -172,29 +165,89 @@ delta_rule_kernel(DeltaArgs A) {
       const float kinv = FAST ? __builtin_amdgcn_rsqf(kk + A.unit_eps) : 1.0f / sqrtf(kk + A.unit_eps);
       for (int d = lane; d < DP; d += DA_WAVE) { at[d] *= qinv; at[DP + d] *= kinv; }
     }
-    __syncthreads();
+    lds_barrier();
+    // what a four's walk takes, in place: q <- G_t q, k <- G_t k, g <- P_4t k; G_4, A and B beside
+    for (int f = wave; f < n_fours; f += 256 / DA_WAVE) {
+      float ab[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ab[i] = 0.f;
+      for (int d = lane; d < DP; d += DA_WAVE) {
+        float* t0 = stage + (f * 4) * TS + d;
+        float q[4], k[4], g[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) { q[t] = t0[t * TS]; k[t] = t0[t * TS + DP]; g[t] = t0[t * TS + 2 * DP]; }
+        const float p21 = g[1], p32 = g[2], p43 = g[3], p31 = g[1] * g[2], p42 = g[2] * g[3], p41 = p31 * g[3];
+        const float G1 = g[0], G2 = G1 * g[1], G3 = G2 * g[2], G4 = G3 * g[3];
+        ab[0] = fmaf(k[1] * k[0], p21, ab[0]);                   // A21 A31 A32 A41 A42 A43
+        ab[1] = fmaf(k[2] * k[0], p31, ab[1]);
+        ab[2] = fmaf(k[2] * k[1], p32, ab[2]);
+        ab[3] = fmaf(k[3] * k[0], p41, ab[3]);
+        ab[4] = fmaf(k[3] * k[1], p42, ab[4]);
+        ab[5] = fmaf(k[3] * k[2], p43, ab[5]);
+        ab[6] = fmaf(q[0], k[0], ab[6]);                         // B11 | B21 B22 | B31 B32 B33 | B41 B42 B43 B44
+        ab[7] = fmaf(q[1] * k[0], p21, ab[7]);
+        ab[8] = fmaf(q[1], k[1], ab[8]);
+        ab[9] = fmaf(q[2] * k[0], p31, ab[9]);
+        ab[10] = fmaf(q[2] * k[1], p32, ab[10]);
+        ab[11] = fmaf(q[2], k[2], ab[11]);
+        ab[12] = fmaf(q[3] * k[0], p41, ab[12]);
+        ab[13] = fmaf(q[3] * k[1], p42, ab[13]);
+        ab[14] = fmaf(q[3] * k[2], p43, ab[14]);
+        ab[15] = fmaf(q[3], k[3], ab[15]);
+        t0[0] = q[0] * G1;          t0[DP] = k[0] * G1;          t0[2 * DP] = k[0] * p41;
+        t0[TS] = q[1] * G2;         t0[TS + DP] = k[1] * G2;     t0[TS + 2 * DP] = k[1] * p42;
+        t0[2 * TS] = q[2] * G3;     t0[2 * TS + DP] = k[2] * G3; t0[2 * TS + 2 * DP] = k[2] * p43;
+        t0[3 * TS] = q[3] * G4;     t0[3 * TS + DP] = k[3] * G4; t0[3 * TS + 2 * DP] = k[3];
+        fours[f * FS + d] = G4;
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) ab[i] = wave_sum(ab[i]);
+      if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) fours[f * FS + DP + i] = ab[i];
+      }
+    }
+    lds_barrier();
     if (n0 + TB < last) fetch(n0 + TB);              // in flight while this block is walked
-    DeltaToken<RPL> cur, nxt;
-    take(0, cur);
-    for (int tok = 0; tok < cnt; ++tok) {
-      take(tok + 1 < TB ? tok + 1 : tok, nxt);       // the next token's numbers, ahead
-      float dot = 0.f;
+    for (int f = 0; f < n_fours; ++f) {
+      const float* t0 = stage + (f * 4) * TS;
+      const float* fd = fours + f * FS;
+      float dk[4], eq[4], v[4], be[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        dk[t] = 0.f; eq[t] = 0.f;
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+          dk[t] = fmaf(S[r], t0[t * TS + DP + row0 + r], dk[t]);
+          eq[t] = fmaf(S[r], t0[t * TS + row0 + r], eq[t]);
+        }
+        v[t] = t0[t * TS + 3 * DP + tid / DELTA_LPC];
+        be[t] = t0[t * TS + 3 * DP + DELTA_CPB];
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t) { dk[t] = group_sum<DELTA_LPC>(dk[t]); eq[t] = group_sum<DELTA_LPC>(eq[t]); }
+      const float* ab = fd + DP;
+      const float u0 = be[0] * (v[0] - dk[0]);
+      const float u1 = be[1] * (v[1] - dk[1] - ab[0] * u0);
+      const float u2 = be[2] * (v[2] - dk[2] - ab[1] * u0 - ab[2] * u1);
+      const float u3 = be[3] * (v[3] - dk[3] - ab[3] * u0 - ab[4] * u1 - ab[5] * u2);
+      const float o0 = eq[0] + ab[6] * u0;
+      const float o1 = eq[1] + ab[7] * u0 + ab[8] * u1;
+      const float o2 = eq[2] + ab[9] * u0 + ab[10] * u1 + ab[11] * u2;
+      const float o3 = eq[3] + ab[12] * u0 + ab[13] * u1 + ab[14] * u2 + ab[15] * u3;
 #pragma unroll
       for (int r = 0; r < RPL; ++r) {
-        S[r] *= A.channel ? cur.g[r] : cur.gh;
-        dot = fmaf(S[r], cur.k[r], dot);
+        float x = fd[row0 + r] * S[r];
+        x = fmaf(t0[2 * DP + row0 + r], u0, x);
+        x = fmaf(t0[TS + 2 * DP + row0 + r], u1, x);
+        x = fmaf(t0[2 * TS + 2 * DP + row0 + r], u2, x);
+        x = fmaf(t0[3 * TS + 2 * DP + row0 + r], u3, x);
+        S[r] = x;
       }
-      dot = group_sum<DELTA_LPC>(dot);
-      const float u = cur.b * (cur.v - dot);
-      float out = 0.f;
-#pragma unroll
-      for (int r = 0; r < RPL; ++r) {
-        S[r] = fmaf(cur.k[r], u, S[r]);
-        out = fmaf(S[r], cur.q[r], out);
-      }
-      out = group_sum<DELTA_LPC>(out);
-      if (sub == 0 && col_ok) A.o[(size_t)(n0 + tok) * A.o_ld + h * A.Dv + col] = out;
-      cur = nxt;
+      // lanes 0..3 of a column's 16 write its four read-outs
+      const int tok = f * 4 + sub;
+      if (sub < 4 && tok < cnt && col_ok)
+        A.o[(size_t)(n0 + tok) * A.o_ld + h * A.Dv + col] = sub == 0 ? o0 : (sub == 1 ? o1 : (sub == 2 ? o2 : o3));
     }
   }
   if (srow && col_ok && A.write) {
