@@ -73,8 +73,10 @@ attn_window_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
   aw_bf16x8_t qf[D16];
 #pragma unroll
   for (int kd = 0; kd < D16; ++kd) {
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (q_ok && kd * 16 + hf * 8 < D) v = *(const uint4*)(q + (size_t)(row0 + qi) * q_ld + h * D + kd * 16 + hf * 8);
+    // (unconditional, from a row and a place that exist, replaced afterwards: see the keys' loads below)
+    const int off = kd * 16 + hf * 8;
+    uint4 v = *(const uint4*)(q + (size_t)(row0 + (qi < T ? qi : T - 1)) * q_ld + h * D + (off < D ? off : 0));
+    if (!q_ok || off >= D) v = make_uint4(0, 0, 0, 0);
     qf[kd] = __builtin_bit_cast(aw_bf16x8_t, v);
   }
   // the wavefront's rows span positions w_first .. w_last; its keys are w_lo .. w_last and those below kfw
@@ -106,10 +108,13 @@ attn_window_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     {
       const int j = kt + col, jj = (whole || key_ok(j)) ? j : safe_key;
       const bf16_t* kr = kbase + page_of(jj) + (long long)(jj & pmask) * D;
+      // (unconditional loads, replaced afterwards where the head has no such entries: a load under a condition
+      // becomes a branch, and the loads would wait for each other)
 #pragma unroll
       for (int kd = 0; kd < D16; ++kd) {
-        uint4 v = make_uint4(0, 0, 0, 0);
-        if (kd * 16 + hf * 8 < D) v = *(const uint4*)(kr + kd * 16 + hf * 8);
+        const int off = kd * 16 + hf * 8;
+        uint4 v = *(const uint4*)(kr + (off < D ? off : 0));
+        if (off >= D) v = make_uint4(0, 0, 0, 0);
         tl.k[kd] = v;
       }
     }

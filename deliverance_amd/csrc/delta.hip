@@ -10,7 +10,7 @@
 //
 // The columns of S do not meet: column j needs k, q, g, beta and v[j] only.  A column is shared out over 16
 // neighbouring lanes, each with RPL consecutive rows in registers; the two sums over rows are taken inside the
-// lane and then over the 16 lanes by DPP additions.  A wavefront holds 4 columns, a workgroup of 4 wavefronts 16;
+// lane and then over the 16 lanes by DPP additions.  A wavefront holds 4 columns, a workgroup's 4 walking wavefronts 16;
 // the grid is (sequences x heads x column blocks), each walking its sequence's portion in order; the tokens' numbers
 // come through LDS in blocks (see the kernel).  The order of every sum depends on D only, so a token's result
 // does not depend on how the sequence was cut into steps or on its neighbours in the batch.
@@ -56,162 +56,169 @@ struct DeltaArgs {
   float unit_eps, q_scale;
 };
 
-// Tokens come through LDS in blocks of TB: the whole workgroup loads a block (every number once, coalesced) and
-// turns the raw numbers into what the recurrence takes; the next block's loads are in flight while this one is
-// walked.  The walk itself goes four tokens at a time.  With S the state in front of tokens 1..4, P_ts the product
-// of the decays of tokens s+1..t (row by row; P_tt = 1) and G_t = P_t0 the product of the decays of tokens 1..t:
+// Tokens come through LDS in blocks of TB, and a workgroup is two teams of four wavefronts.  The walkers hold the
+// state (16 columns, a column over 16 lanes) and walk a block four tokens at a time; meanwhile the helpers make the
+// next block ready in the other LDS buffer: a helper takes whole fours, loads their raw numbers (every load
+// unconditional, from a place that exists), and works out in registers, a lane a key row, everything that does not
+// depend on the state.  One barrier a block.  With S the state in front of tokens 1..4, P_ts the product of the decays
+// of tokens s+1..t (row by row; P_tt = 1) and G_t = P_t0 the product of the decays of tokens 1..t:
 //     u_t = beta_t (v_t - S^T (G_t k_t) - sum_{s<t} A_ts u_s)        A_ts = sum_d k_t k_s P_ts
 //     o_t = S^T (G_t q_t) + sum_{s<=t} B_ts u_s                       B_ts = sum_d q_t k_s P_ts
 //     S  <- G_4 S + sum_s (P_4s k_s) u_s^T
 // which is the token-by-token rule written out (no quotient of decays anywhere: only products of numbers in (0, 1]).
-// A, B, G_t k_t, G_t q_t and P_4s k_s do not depend on the state: wavefronts work them out for the block's fours
-// side by side.  What is left on the path from one four's state to the next: eight sums over the rows of a column
-// (independent of each other, so their lane exchanges overlap), ten multiply-adds on a column's four u, and the
-// update.  A portion's last four is filled up with tokens that change nothing (decay 1, beta 0, k = q = 0).
-template <typename T, int RPL, bool FAST>
-__global__ void __launch_bounds__(256)
+// The helpers leave G_t q_t, G_t k_t, P_4s k_s, G_4, A, B, beta and the columns' values.  What is left on the path
+// from one four's state to the next: eight sums over the rows of a column (independent of each other, so their lane
+// exchanges overlap), ten multiply-adds on a column's four u, and the update.  A portion's last four is filled up
+// with tokens that change nothing (decay 1, beta 0, k = q = 0).
+#define DELTA_TEAM 256        // threads of a team
+// SHORT: no sequence brings more than four tokens (decoding): one four a block, one buffer, one helping wavefront.
+template <typename T, int RPL, bool FAST, bool SHORT>
+__global__ void __launch_bounds__(2 * DELTA_TEAM)
 delta_rule_kernel(DeltaArgs A) {
   constexpr int DP = RPL * DELTA_LPC;                        // key rows, padded
-  constexpr int TB = RPL <= 4 ? 32 : (RPL == 8 ? 16 : 8);    // tokens a block
-  constexpr int TS = 3 * DP + 20;                            // floats a token: q | k | g | 16 values | beta
+  constexpr int TB = SHORT ? 4 : (RPL <= 4 ? 32 : (RPL == 8 ? 16 : 8));    // tokens a block
+  constexpr int NBUF = SHORT ? 1 : 2;
+  constexpr int TS = 3 * DP + 20;                            // floats a token: G q | G k | P k | 16 values | beta
   constexpr int NF = TB / 4, FS = DP + 16;                   // fours a block; floats a four: G_4 | A (6) | B (10)
-  constexpr int PT = (TB * DP + 255) / 256, PV = (TB * DELTA_CPB + 255) / 256;
-  __shared__ __attribute__((aligned(16))) float stage[TB * TS];
-  __shared__ __attribute__((aligned(16))) float fours[NF * FS];
+  constexpr int EL = (DP + DA_WAVE - 1) / DA_WAVE;           // key rows a helper's lane
+  __shared__ __attribute__((aligned(16))) float stage[NBUF][TB * TS];
+  __shared__ __attribute__((aligned(16))) float fours[NBUF][NF * FS];
   const int blocks_per_head = (A.Dv + DELTA_CPB - 1) / DELTA_CPB;
   const int cb = blockIdx.x % blocks_per_head;
   const int h = (blockIdx.x / blocks_per_head) % A.H;
   const int s = blockIdx.x / (blocks_per_head * A.H);
   const int kh = h / (A.H / A.G);
-  const int tid = threadIdx.x, lane = tid % DA_WAVE, wave = tid / DA_WAVE;
+  const int tid = threadIdx.x % DELTA_TEAM, lane = tid % DA_WAVE;
+  const bool helper = threadIdx.x >= DELTA_TEAM;             // (the same for a whole wavefront)
+  const int hw = tid / DA_WAVE;                              // the wavefront's number in its team
   const int sub = tid % DELTA_LPC;
   const int col = cb * DELTA_CPB + tid / DELTA_LPC;
   const bool col_ok = col < A.Dv;
   const int row0 = sub * RPL;
   const int first = A.q_start[s], last = A.q_start[s + 1];
-  const int slot = A.state_slots[s];
-  float* srow = slot >= 0 ? A.state + (size_t)slot * A.state_ld + ((size_t)h * A.Dv + (col_ok ? col : 0)) * A.D : nullptr;
+  const int n_blocks = (last - first + TB - 1) / TB;
   const float rate = A.rate[h];
 
-  float S[RPL];
-#pragma unroll
-  for (int r = 0; r < RPL; ++r) S[r] = (srow && col_ok && row0 + r < A.D) ? srow[row0 + r] : 0.f;
-
-  // a thread's share of a block, from memory into registers
-  float rq[PT], rk[PT], ra[PT], rv[PV], rb = 0.f;
-  // (every load is unconditional, from a place that exists, and what does not count is replaced afterwards: a load
-  // under a condition becomes a branch, and the loads would wait for each other)
-  auto fetch = [&](int n0) {
+  // a helper: fours hw, hw + 4, ... of block b, from memory to the block's LDS buffer
+  auto prepare = [&](int b) {
+    const int n0 = first + b * TB;
     const int cnt = last - n0 < TB ? last - n0 : TB;
+    float* st = stage[b & (NBUF - 1)];
+    float* fo = fours[b & (NBUF - 1)];
+    for (int f = hw; f * 4 < cnt; f += DELTA_TEAM / DA_WAVE) {
+      float q[EL][4], k[EL][4], g[EL][4], vv[4];
 #pragma unroll
-    for (int i = 0; i < PT; ++i) {
-      const int idx = tid + i * 256, tok = idx / DP, d = idx % DP;
-      const bool ok = tok < cnt && d < A.D;
-      const int tc = tok < cnt ? tok : cnt - 1, dc = d < A.D ? d : A.D - 1;
-      const T* row = (const T*)A.qkv + (size_t)(n0 + tc) * A.ld;
-      const int ac = A.channel ? h * A.D + dc : h;
-      const float xq = to_f32(row[kh * A.D + dc]), xk = to_f32(row[A.k_off + kh * A.D + dc]);
-      const float xa = A.araw[(size_t)(n0 + tc) * A.a_ld + A.a_off + ac] + A.dt_bias[ac];
-      rq[i] = ok ? xq : 0.f;
-      rk[i] = ok ? xk : 0.f;
-      ra[i] = ok ? xa : 0.f;
-    }
+      for (int t = 0; t < 4; ++t) {
+        const int tok = f * 4 + t, tc = tok < cnt ? tok : cnt - 1;
+        const T* row = (const T*)A.qkv + (size_t)(n0 + tc) * A.ld;
 #pragma unroll
-    for (int i = 0; i < PV; ++i) {
-      const int idx = (tid + i * 256) % (TB * DELTA_CPB), tok = idx / DELTA_CPB, c = cb * DELTA_CPB + idx % DELTA_CPB;
-      const bool ok = tok < cnt && c < A.Dv;
-      const int tc = tok < cnt ? tok : cnt - 1, cc = c < A.Dv ? c : A.Dv - 1;
-      const float xv = to_f32(((const T*)A.qkv)[(size_t)(n0 + tc) * A.ld + A.v_off + h * A.Dv + cc]);
-      rv[i] = ok ? xv : 0.f;
-    }
-    rb = A.braw[(size_t)(n0 + (tid < cnt ? tid : cnt - 1)) * A.b_ld + h];
-  };
-  // ... and from registers into LDS, the decays and beta worked out on the way; tokens past the block's last and
-  // rows past D change nothing
-  auto park = [&](int cnt) {
-#pragma unroll
-    for (int i = 0; i < PT; ++i) {
-      const int idx = tid + i * 256, tok = idx / DP, d = idx % DP;
-      if (PT * 256 == TB * DP || idx < TB * DP) {
-        float* at = stage + tok * TS + d;
-        at[0] = rq[i];
-        at[DP] = rk[i];
-        at[2 * DP] = (tok < cnt && d < A.D) ? delta_exp<FAST>(-rate * delta_softplus<FAST>(ra[i])) : 1.f;
+        for (int e = 0; e < EL; ++e) {
+          const int d = lane + e * DA_WAVE, dc = d < A.D ? d : A.D - 1;
+          const int ac = A.channel ? h * A.D + dc : h;
+          q[e][t] = to_f32(row[kh * A.D + dc]);
+          k[e][t] = to_f32(row[A.k_off + kh * A.D + dc]);
+          g[e][t] = A.araw[(size_t)(n0 + tc) * A.a_ld + A.a_off + ac] + A.dt_bias[ac];
+        }
+        const int c = cb * DELTA_CPB + lane % DELTA_CPB;
+        vv[t] = to_f32(row[A.v_off + h * A.Dv + (c < A.Dv ? c : A.Dv - 1)]);
       }
-    }
+      const int bt = f * 4 + lane % 4;                         // the token whose beta this lane takes
+      const float braw = A.braw[(size_t)(n0 + (bt < cnt ? bt : cnt - 1)) * A.b_ld + h];
+      // q and k to unit length (q also times D^-1/2), decays; tokens past the block's last and rows past D change nothing
 #pragma unroll
-    for (int i = 0; i < PV; ++i) {
-      const int idx = tid + i * 256;
-      if (idx < TB * DELTA_CPB) stage[(idx / DELTA_CPB) * TS + 3 * DP + idx % DELTA_CPB] = rv[i];
-    }
-    if (tid < TB) stage[tid * TS + 3 * DP + DELTA_CPB] = tid < cnt ? delta_logistic<FAST>(rb) : 0.f;
-  };
-
-  if (first < last) fetch(first);
-  for (int n0 = first; n0 < last; n0 += TB) {
-    const int cnt = last - n0 < TB ? last - n0 : TB;
-    const int n_fours = (cnt + 3) / 4;
-    lds_barrier();                                   // the block before has been walked (its stores may still be on their way)
-    park(cnt);
-    lds_barrier();
-    // q and k to unit length (q also times D^-1/2): wavefront w takes tokens w, w + 4, ...
-    for (int tok = wave; tok < cnt; tok += 256 / DA_WAVE) {
-      float* at = stage + tok * TS;
-      float qq = 0.f, kk = 0.f;
-      for (int d = lane; d < DP; d += DA_WAVE) { qq = fmaf(at[d], at[d], qq); kk = fmaf(at[DP + d], at[DP + d], kk); }
-      qq = wave_sum(qq);
-      kk = wave_sum(kk);
-      const float qinv = (FAST ? __builtin_amdgcn_rsqf(qq + A.unit_eps) : 1.0f / sqrtf(qq + A.unit_eps)) * A.q_scale;
-      const float kinv = FAST ? __builtin_amdgcn_rsqf(kk + A.unit_eps) : 1.0f / sqrtf(kk + A.unit_eps);
-      for (int d = lane; d < DP; d += DA_WAVE) { at[d] *= qinv; at[DP + d] *= kinv; }
-    }
-    lds_barrier();
-    // what a four's walk takes, in place: q <- G_t q, k <- G_t k, g <- P_4t k; G_4, A and B beside
-    for (int f = wave; f < n_fours; f += 256 / DA_WAVE) {
+      for (int t = 0; t < 4; ++t) {
+        const bool tok_ok = f * 4 + t < cnt;
+        float qq = 0.f, kk = 0.f;
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+          const bool ok = tok_ok && lane + e * DA_WAVE < A.D;
+          q[e][t] = ok ? q[e][t] : 0.f;
+          k[e][t] = ok ? k[e][t] : 0.f;
+          g[e][t] = ok ? delta_exp<FAST>(-rate * delta_softplus<FAST>(g[e][t])) : 1.f;
+          qq = fmaf(q[e][t], q[e][t], qq);
+          kk = fmaf(k[e][t], k[e][t], kk);
+        }
+        qq = wave_sum(qq);
+        kk = wave_sum(kk);
+        const float qinv = (FAST ? __builtin_amdgcn_rsqf(qq + A.unit_eps) : 1.0f / sqrtf(qq + A.unit_eps)) * A.q_scale;
+        const float kinv = FAST ? __builtin_amdgcn_rsqf(kk + A.unit_eps) : 1.0f / sqrtf(kk + A.unit_eps);
+#pragma unroll
+        for (int e = 0; e < EL; ++e) { q[e][t] *= qinv; k[e][t] *= kinv; }
+      }
       float ab[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) ab[i] = 0.f;
-      for (int d = lane; d < DP; d += DA_WAVE) {
-        float* t0 = stage + (f * 4) * TS + d;
-        float q[4], k[4], g[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) { q[t] = t0[t * TS]; k[t] = t0[t * TS + DP]; g[t] = t0[t * TS + 2 * DP]; }
-        const float p21 = g[1], p32 = g[2], p43 = g[3], p31 = g[1] * g[2], p42 = g[2] * g[3], p41 = p31 * g[3];
-        const float G1 = g[0], G2 = G1 * g[1], G3 = G2 * g[2], G4 = G3 * g[3];
-        ab[0] = fmaf(k[1] * k[0], p21, ab[0]);                   // A21 A31 A32 A41 A42 A43
-        ab[1] = fmaf(k[2] * k[0], p31, ab[1]);
-        ab[2] = fmaf(k[2] * k[1], p32, ab[2]);
-        ab[3] = fmaf(k[3] * k[0], p41, ab[3]);
-        ab[4] = fmaf(k[3] * k[1], p42, ab[4]);
-        ab[5] = fmaf(k[3] * k[2], p43, ab[5]);
-        ab[6] = fmaf(q[0], k[0], ab[6]);                         // B11 | B21 B22 | B31 B32 B33 | B41 B42 B43 B44
-        ab[7] = fmaf(q[1] * k[0], p21, ab[7]);
-        ab[8] = fmaf(q[1], k[1], ab[8]);
-        ab[9] = fmaf(q[2] * k[0], p31, ab[9]);
-        ab[10] = fmaf(q[2] * k[1], p32, ab[10]);
-        ab[11] = fmaf(q[2], k[2], ab[11]);
-        ab[12] = fmaf(q[3] * k[0], p41, ab[12]);
-        ab[13] = fmaf(q[3] * k[1], p42, ab[13]);
-        ab[14] = fmaf(q[3] * k[2], p43, ab[14]);
-        ab[15] = fmaf(q[3], k[3], ab[15]);
-        t0[0] = q[0] * G1;          t0[DP] = k[0] * G1;          t0[2 * DP] = k[0] * p41;
-        t0[TS] = q[1] * G2;         t0[TS + DP] = k[1] * G2;     t0[TS + 2 * DP] = k[1] * p42;
-        t0[2 * TS] = q[2] * G3;     t0[2 * TS + DP] = k[2] * G3; t0[2 * TS + 2 * DP] = k[2] * p43;
-        t0[3 * TS] = q[3] * G4;     t0[3 * TS + DP] = k[3] * G4; t0[3 * TS + 2 * DP] = k[3];
-        fours[f * FS + d] = G4;
+      for (int e = 0; e < EL; ++e) {
+        const int d = lane + e * DA_WAVE;
+        const float* qe = q[e];
+        const float* ke = k[e];
+        const float* ge = g[e];
+        const float p21 = ge[1], p32 = ge[2], p43 = ge[3], p31 = ge[1] * ge[2], p42 = ge[2] * ge[3], p41 = p31 * ge[3];
+        const float G1 = ge[0], G2 = G1 * ge[1], G3 = G2 * ge[2], G4 = G3 * ge[3];
+        ab[0] = fmaf(ke[1] * ke[0], p21, ab[0]);                 // A21 A31 A32 A41 A42 A43
+        ab[1] = fmaf(ke[2] * ke[0], p31, ab[1]);
+        ab[2] = fmaf(ke[2] * ke[1], p32, ab[2]);
+        ab[3] = fmaf(ke[3] * ke[0], p41, ab[3]);
+        ab[4] = fmaf(ke[3] * ke[1], p42, ab[4]);
+        ab[5] = fmaf(ke[3] * ke[2], p43, ab[5]);
+        ab[6] = fmaf(qe[0], ke[0], ab[6]);                       // B11 | B21 B22 | B31 B32 B33 | B41 B42 B43 B44
+        ab[7] = fmaf(qe[1] * ke[0], p21, ab[7]);
+        ab[8] = fmaf(qe[1], ke[1], ab[8]);
+        ab[9] = fmaf(qe[2] * ke[0], p31, ab[9]);
+        ab[10] = fmaf(qe[2] * ke[1], p32, ab[10]);
+        ab[11] = fmaf(qe[2], ke[2], ab[11]);
+        ab[12] = fmaf(qe[3] * ke[0], p41, ab[12]);
+        ab[13] = fmaf(qe[3] * ke[1], p42, ab[13]);
+        ab[14] = fmaf(qe[3] * ke[2], p43, ab[14]);
+        ab[15] = fmaf(qe[3], ke[3], ab[15]);
+        if (d < DP) {
+          float* t0 = st + (f * 4) * TS + d;
+          t0[0] = qe[0] * G1;          t0[DP] = ke[0] * G1;          t0[2 * DP] = ke[0] * p41;
+          t0[TS] = qe[1] * G2;         t0[TS + DP] = ke[1] * G2;     t0[TS + 2 * DP] = ke[1] * p42;
+          t0[2 * TS] = qe[2] * G3;     t0[2 * TS + DP] = ke[2] * G3; t0[2 * TS + 2 * DP] = ke[2] * p43;
+          t0[3 * TS] = qe[3] * G4;     t0[3 * TS + DP] = ke[3] * G4; t0[3 * TS + 2 * DP] = ke[3];
+          fo[f * FS + d] = G4;
+        }
       }
 #pragma unroll
       for (int i = 0; i < 16; ++i) ab[i] = wave_sum(ab[i]);
       if (lane == 0) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) fours[f * FS + DP + i] = ab[i];
+        for (int i = 0; i < 16; ++i) fo[f * FS + DP + i] = ab[i];
       }
+      if (lane < DELTA_CPB) {
+        const bool c_ok = cb * DELTA_CPB + lane < A.Dv;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) st[(f * 4 + t) * TS + 3 * DP + lane] = (c_ok && f * 4 + t < cnt) ? vv[t] : 0.f;
+      }
+      if (lane < 4) st[(f * 4 + lane) * TS + 3 * DP + DELTA_CPB] = bt < cnt ? delta_logistic<FAST>(braw) : 0.f;
     }
+  };
+
+  if (helper) {
+    if (n_blocks > 0) prepare(0);
     lds_barrier();
-    if (n0 + TB < last) fetch(n0 + TB);              // in flight while this block is walked
+    for (int b = 0; b < n_blocks; ++b) {
+      if (b + 1 < n_blocks) prepare(b + 1);
+      lds_barrier();
+    }
+    return;
+  }
+
+  const int slot = A.state_slots[s];
+  float* srow = slot >= 0 ? A.state + (size_t)slot * A.state_ld + ((size_t)h * A.Dv + (col_ok ? col : 0)) * A.D : nullptr;
+  float S[RPL];
+#pragma unroll
+  for (int r = 0; r < RPL; ++r) S[r] = (srow && col_ok && row0 + r < A.D) ? srow[row0 + r] : 0.f;
+  lds_barrier();
+  for (int b = 0; b < n_blocks; ++b) {
+    const int n0 = first + b * TB;
+    const int cnt = last - n0 < TB ? last - n0 : TB;
+    const int n_fours = (cnt + 3) / 4;
     for (int f = 0; f < n_fours; ++f) {
-      const float* t0 = stage + (f * 4) * TS;
-      const float* fd = fours + f * FS;
+      const float* t0 = stage[b & (NBUF - 1)] + (f * 4) * TS;
+      const float* fd = fours[b & (NBUF - 1)] + f * FS;
       float dk[4], eq[4], v[4], be[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
@@ -249,6 +256,7 @@ delta_rule_kernel(DeltaArgs A) {
       if (sub < 4 && tok < cnt && col_ok)
         A.o[(size_t)(n0 + tok) * A.o_ld + h * A.Dv + col] = sub == 0 ? o0 : (sub == 1 ? o1 : (sub == 2 ? o2 : o3));
     }
+    lds_barrier();
   }
   if (srow && col_ok && A.write) {
 #pragma unroll
@@ -258,10 +266,15 @@ delta_rule_kernel(DeltaArgs A) {
 }
 
 template <typename T, bool FAST>
-static int delta_launch(const DeltaArgs& A, int S, void* stream) {
+static int delta_launch(const DeltaArgs& A, int S, int max_rows, void* stream) {
   const int rpl = (A.D + DELTA_LPC - 1) / DELTA_LPC;
-  const dim3 grid((unsigned)(S * A.H * ((A.Dv + DELTA_CPB - 1) / DELTA_CPB))), block(256);
-#define DA_DELTA_GO(R) hipLaunchKernelGGL((delta_rule_kernel<T, R, FAST>), grid, block, 0, (hipStream_t)stream, A)
+  const bool brief = max_rows > 0 && max_rows <= 4;
+  const dim3 grid((unsigned)(S * A.H * ((A.Dv + DELTA_CPB - 1) / DELTA_CPB))), block(brief ? DELTA_TEAM + DA_WAVE : 2 * DELTA_TEAM);
+#define DA_DELTA_GO(R)                                                                                          \
+  do {                                                                                                          \
+    if (brief) hipLaunchKernelGGL((delta_rule_kernel<T, R, FAST, true>), grid, block, 0, (hipStream_t)stream, A); \
+    else hipLaunchKernelGGL((delta_rule_kernel<T, R, FAST, false>), grid, block, 0, (hipStream_t)stream, A);    \
+  } while (0)
   if (rpl <= 1) DA_DELTA_GO(1);
   else if (rpl <= 2) DA_DELTA_GO(2);
   else if (rpl <= 4) DA_DELTA_GO(4);
@@ -272,10 +285,11 @@ static int delta_launch(const DeltaArgs& A, int S, void* stream) {
   return 0;
 }
 
+// max_rows: the most tokens a sequence of the step brings (0: not known)
 extern "C" int da_delta_rule(const void* qkv, int dtype, int ld, int k_off, int v_off, const float* braw, int b_ld,
                              const float* araw, int a_ld, int a_off, const float* dt_bias, const float* rate, float* state,
                              long state_ld, const int* state_slots, const int* q_start, float* o, int o_ld, int S, int H,
-                             int G, int D, int Dv, int channel, float unit_eps, int write, void* stream) {
+                             int G, int D, int Dv, int channel, float unit_eps, int write, int max_rows, void* stream) {
   DA_REQUIRE(S >= 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0, "delta_rule: bad sizes");
   DA_REQUIRE(D <= DELTA_MAX_D, "delta_rule: a key size of %d, %d are taken", D, DELTA_MAX_D);
   DA_REQUIRE(k_off >= G * D && v_off >= k_off + G * D && ld >= v_off + H * Dv, "delta_rule: q, k and v leave the row");
@@ -288,8 +302,8 @@ extern "C" int da_delta_rule(const void* qkv, int dtype, int ld, int k_off, int 
   A.dt_bias = dt_bias; A.rate = rate; A.state = state; A.state_ld = state_ld; A.state_slots = state_slots;
   A.q_start = q_start; A.o = o; A.o_ld = o_ld; A.H = H; A.G = G; A.D = D; A.Dv = Dv; A.channel = channel; A.write = write;
   A.unit_eps = unit_eps; A.q_scale = 1.0f / sqrtf((float)D);
-  if (dtype == DA_BF16) return delta_launch<bf16_t, true>(A, S, stream);
-  return delta_launch<float, false>(A, S, stream);
+  if (dtype == DA_BF16) return delta_launch<bf16_t, true>(A, S, max_rows, stream);
+  return delta_launch<float, false>(A, S, max_rows, stream);
 }
 
 // One wavefront per (token, head): the read-out divided by its root mean square, times the gain, times the gate.

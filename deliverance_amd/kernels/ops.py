@@ -102,7 +102,7 @@ _ARGTYPES = {
     "da_attn_window_takes": [_I, _I, _I],
     "da_attn_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _I, _VP, _VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _I, _VP],
     "da_delta_rule": [_VP, _I, _I, _I, _I, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I,
-                      _I, _I, _F, _I, _VP],
+                      _I, _I, _F, _I, _I, _VP],
     "da_delta_gate_norm": [_VP, _I, _VP, _I, _I, _VP, _I, _F, _I, _VP, _I, _I, _I, _I, _VP],
     "da_scale_add_rows": [_VP, _VP, _VP, _I, _I, _F, _VP],
     "da_kv_write_split": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
@@ -1532,7 +1532,8 @@ def delta_rule(ctx, qkv: torch.Tensor, k_off: int, v_off: int, beta_raw: torch.T
         _check(_lib().da_delta_rule(_ptr(qkv), _dt(qkv), qkv.stride(0), k_off, v_off, _ptr(beta_raw), beta_raw.stride(0),
                                     _ptr(decay_raw), decay_raw.stride(0), int(decay_off), _ptr(dt_bias), _ptr(rate), _ptr(state), ld,
                                     _ptr(ctx.state_slots), _ptr(ctx.q_start), _ptr(o), o.stride(0), ctx.n_seqs, H, G, D, Dv,
-                                    int(bool(channel_decay)), float(unit_eps), int(bool(write)), _stream()))
+                                    int(bool(channel_decay)), float(unit_eps), int(bool(write)),
+                                    int(getattr(ctx, "max_query_len", 0) or 0), _stream()))
     return o
 
 

@@ -145,7 +145,12 @@ class ExpertsFeedForward(FeedForward):
                             self.weight, self.activation, x, accumulate=ctx.part_accumulate, ids=ids,
                             pair_weights=weights, gated=self.gated, weight_input=self.weight_on == "input")
         if self.shared is not None:
-            self.shared.forward(ctx, h, x)
+            keep = ctx.part_accumulate
+            ctx.part_accumulate = True          # the shared expert joins the experts' sum, stored or added above
+            try:
+                self.shared.forward(ctx, h, x)
+            finally:
+                ctx.part_accumulate = keep
 
 
 register_feed_forward("gated", GatedFeedForward)
