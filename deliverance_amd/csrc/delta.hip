@@ -56,7 +56,8 @@ struct DeltaArgs {
   float unit_eps, q_scale;
 };
 
-// Tokens come through LDS in blocks of TB, and a workgroup is two teams of four wavefronts.  The walkers hold the
+// Tokens come through LDS in blocks of TB, and a workgroup is two teams: four walking wavefronts and up to eight
+// helping ones.  The walkers hold the
 // state (16 columns, a column over 16 lanes) and walk a block four tokens at a time; meanwhile the helpers make the
 // next block ready in the other LDS buffer: a helper takes whole fours, loads their raw numbers (every load
 // unconditional, from a place that exists), and works out in registers, a lane a key row, everything that does not
@@ -70,10 +71,12 @@ struct DeltaArgs {
 // from one four's state to the next: eight sums over the rows of a column (independent of each other, so their lane
 // exchanges overlap), ten multiply-adds on a column's four u, and the update.  A portion's last four is filled up
 // with tokens that change nothing (decay 1, beta 0, k = q = 0).
-#define DELTA_TEAM 256        // threads of a team
+#define DELTA_TEAM 256        // threads that walk
+#define DELTA_HELPERS 8       // helping wavefronts: one a four of a block of 32 tokens (a four is a trip to memory and
+                              // some arithmetic; two fours a helper in a row took as long as the walk of the block)
 // SHORT: no sequence brings more than four tokens (decoding): one four a block, one buffer, one helping wavefront.
 template <typename T, int RPL, bool FAST, bool SHORT>
-__global__ void __launch_bounds__(2 * DELTA_TEAM)
+__global__ void __launch_bounds__(DELTA_TEAM + DELTA_HELPERS * DA_WAVE)
 delta_rule_kernel(DeltaArgs A) {
   constexpr int DP = RPL * DELTA_LPC;                        // key rows, padded
   constexpr int TB = SHORT ? 4 : (RPL <= 4 ? 32 : (RPL == 8 ? 16 : 8));    // tokens a block
@@ -88,9 +91,10 @@ delta_rule_kernel(DeltaArgs A) {
   const int h = (blockIdx.x / blocks_per_head) % A.H;
   const int s = blockIdx.x / (blocks_per_head * A.H);
   const int kh = h / (A.H / A.G);
-  const int tid = threadIdx.x % DELTA_TEAM, lane = tid % DA_WAVE;
+  const int tid = threadIdx.x, lane = tid % DA_WAVE;          // (tid: a walker's)
   const bool helper = threadIdx.x >= DELTA_TEAM;             // (the same for a whole wavefront)
-  const int hw = tid / DA_WAVE;                              // the wavefront's number in its team
+  const int hw = ((int)threadIdx.x - DELTA_TEAM) / DA_WAVE;  // a helper's number
+  const int n_helpers = ((int)blockDim.x - DELTA_TEAM) / DA_WAVE;
   const int sub = tid % DELTA_LPC;
   const int col = cb * DELTA_CPB + tid / DELTA_LPC;
   const bool col_ok = col < A.Dv;
@@ -105,7 +109,7 @@ delta_rule_kernel(DeltaArgs A) {
     const int cnt = last - n0 < TB ? last - n0 : TB;
     float* st = stage[b & (NBUF - 1)];
     float* fo = fours[b & (NBUF - 1)];
-    for (int f = hw; f * 4 < cnt; f += DELTA_TEAM / DA_WAVE) {
+    for (int f = hw; f * 4 < cnt; f += n_helpers) {
       float q[EL][4], k[EL][4], g[EL][4], vv[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
@@ -269,7 +273,7 @@ template <typename T, bool FAST>
 static int delta_launch(const DeltaArgs& A, int S, int max_rows, void* stream) {
   const int rpl = (A.D + DELTA_LPC - 1) / DELTA_LPC;
   const bool brief = max_rows > 0 && max_rows <= 4;
-  const dim3 grid((unsigned)(S * A.H * ((A.Dv + DELTA_CPB - 1) / DELTA_CPB))), block(brief ? DELTA_TEAM + DA_WAVE : 2 * DELTA_TEAM);
+  const dim3 grid((unsigned)(S * A.H * ((A.Dv + DELTA_CPB - 1) / DELTA_CPB))), block(DELTA_TEAM + (brief ? 1 : DELTA_HELPERS) * DA_WAVE);
 #define DA_DELTA_GO(R)                                                                                          \
   do {                                                                                                          \
     if (brief) hipLaunchKernelGGL((delta_rule_kernel<T, R, FAST, true>), grid, block, 0, (hipStream_t)stream, A); \

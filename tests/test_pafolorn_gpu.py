@@ -671,7 +671,7 @@ def random_config(seed):
 
     def a_delta(channel):
         G = pick(1, 2, 3)
-        d = delta(G * pick(1, 2, 3), G, pick(8, 16, 24, 33, 64), pick(8, 12, 32, 40), pick(1, 2, 3, 4, 6))
+        d = delta(G * pick(1, 2, 3), G, pick(8, 16, 24, 33, 64, 96, 130), pick(8, 12, 32, 40, 72), pick(1, 2, 3, 4, 6))
         if channel:
             d["a_rank"], d["g_rank"] = pick(1, 4, 9), pick(2, 8, 16)
         return d
@@ -683,8 +683,8 @@ def random_config(seed):
             layers.append(channel_layer(a_delta(True), ff=ff))
         else:
             G = pick(1, 2, 3)
-            D = pick(8, 16, 24, 32, 64)
-            att = attention(G * pick(1, 2, 4), G, D, pick(D, D, 8, 40), float(pick(0.1, D ** -0.5, 0.3)), pick(1, 7, 16, 30, 64),
+            D = pick(8, 16, 24, 32, 64, 48, 128)
+            att = attention(G * pick(1, 2, 4), G, D, pick(D, D, 8, 40, 128), float(pick(0.1, D ** -0.5, 0.3)), pick(1, 7, 16, 30, 64),
                             pick(0, 0, 1, 4, 20), float(pick(100.0, 10000.0, 1e6)), pick(0, D // 2 // 2 * 2, D),
                             softcap=pick(None, 5.0, 30.0))
             layers.append(parallel_layer(att, a_delta(False), float(pick(1.0, 0.7, 1.4)), float(pick(1.0, 0.5, 1.1)), ff=ff))
@@ -693,7 +693,7 @@ def random_config(seed):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(24))
 def test_random_configurations(tmp_path, seed, dtype):
     m = make_model(tmp_path / "m", random_config(seed), 100 + seed)
     ids = m.prompt(75, salt=seed)
