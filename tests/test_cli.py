@@ -54,6 +54,23 @@ def test_random_then_inspect_a_design_with_shared_weights_and_states(tmp_path):
     assert "l0.mix.dkv.norm" in p.stdout and "l1.mix.A_log" in p.stdout and "l1.mlp.shared.down" in p.stdout and "l2." not in p.stdout
 
 
+def test_random_then_inspect_a_design_with_parallel_mixers(tmp_path):
+    """... and on a Pafolorn configuration: a parallel layer keeps two cache slots, a delta rule's low ranks are named."""
+    from pafolorn_models import CONFIG_F
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(CONFIG_F))
+    out = tmp_path / "model"
+    p = run("random", "--config", str(cfg), "--seed", "5", "--out", str(out))
+    assert p.returncode == 0, p.stderr
+    p = run("inspect", str(out))
+    assert p.returncode == 0, p.stderr
+    n = len(CONFIG_F["layers"])
+    slots = sum(2 if L["type"] == "parallel" else 1 for L in CONFIG_F["layers"])
+    assert f"architecture Pafolorn: {n} layers, width {CONFIG_F['width']}, vocabulary {CONFIG_F['vocab']}" in p.stdout
+    assert f"{n} layer calls, {slots} cache slots" in p.stdout
+    assert "l0.mix.left.q.norm" in p.stdout and "l0.mix.right.A_log" in p.stdout and "l0.ls1" in p.stdout and "embed.norm" in p.stdout
+
+
 def test_help_names_the_reference_options():
     p = run("generate", "--help")
     for opt in ("--model", "--working-dtype", "--max-tokens", "--temperature", "--seed", "--warmup-cases", "--max-cases",
