@@ -7,7 +7,7 @@
 // once and the row is read once.
 //
 //   da_rmsnorm      y = rms(x[rows[r]] or x[r])                       (32-bit or bfloat16 out)
-//   da_rmsnorm_add  x += rms_a(src);  h = rms_b(x) (optional)         the norm behind a part, the residual
+//   da_rmsnorm_add  x += rms_a(src);  h = rms_b(x), or x itself converted (optional)   the norm behind a part, the residual
 //                   addition and the norm in front of the next part in one pass over the row
 #include "common.h"
 
@@ -54,7 +54,7 @@ rmsnorm_row_kernel(const float* __restrict__ src, const int* __restrict__ rows, 
     for (int i = 0; i < (EARLY ? VPL : 1); ++i) {
       const int c = (lane + i * DA_WAVE) * 4, cc = c < E ? c : 0;
       ga[i] = rms_param4(wa, wa_dtype, cc);
-      if (ADD && y) gb[i] = rms_param4(wb, wb_dtype, cc);
+      if (ADD && y && wb) gb[i] = rms_param4(wb, wb_dtype, cc);
     }
   }
   float q = 0.f;
@@ -80,7 +80,13 @@ rmsnorm_row_kernel(const float* __restrict__ src, const int* __restrict__ rows, 
       }
     }
   }
-  if (ADD && y) {
+  if (ADD && y && !wb) {                               // no second norm: the new x itself, converted
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+      const int c = (lane + i * DA_WAVE) * 4;
+      if (c < E) rms_store4(y, y_dtype, (size_t)r * E + c, xv[i]);
+    }
+  } else if (ADD && y) {
     const float inv2 = 1.0f / sqrtf(wave_sum(q2) / (float)E + eps);
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
@@ -118,7 +124,9 @@ __global__ void rmsnorm_any_kernel(const float* __restrict__ src, const int* __r
       store_out(y, y_dtype, (size_t)r * E + i, o);
     }
   }
-  if (ADD && y) {
+  if (ADD && y && !wb) {
+    for (int i = lane; i < E; i += DA_WAVE) store_out(y, y_dtype, (size_t)r * E + i, x[(size_t)r * E + i]);
+  } else if (ADD && y) {
     const float inv2 = 1.0f / sqrtf(wave_sum(q2) / (float)E + eps);
     for (int i = lane; i < E; i += DA_WAVE)
       store_out(y, y_dtype, (size_t)r * E + i, x[(size_t)r * E + i] * inv2 * (offset + load_param(wb, wb_dtype, i)));
@@ -163,7 +171,7 @@ extern "C" int da_rmsnorm_add(const float* src, const void* wa, int wa_dtype, fl
   DA_REQUIRE(R >= 0 && E > 0, "rmsnorm_add: bad sizes R=%d E=%d", R, E);
   DA_REQUIRE(eps > 0.f, "rmsnorm_add: eps must be > 0");
   DA_REQUIRE(src && wa && x && (const float*)x != src, "rmsnorm_add: a null operand, or the part's output is the stream itself");
-  DA_REQUIRE((h == nullptr) == (wb == nullptr), "rmsnorm_add: the second norm needs both its gain and its output");
+  DA_REQUIRE(h != nullptr || wb == nullptr, "rmsnorm_add: the second norm needs an output");
   if (R == 0) return 0;
   rms_launch<true>(src, nullptr, wa, wa_dtype, x, wb, wb_dtype, offset, eps, h, h_dtype, R, E, (hipStream_t)stream);
   DA_CHECK_LAUNCH("rmsnorm_add");

@@ -318,15 +318,16 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, gain_offset: float, eps: floa
 def rmsnorm_add(src: torch.Tensor, weight: torch.Tensor, x: torch.Tensor, gain_offset: float, eps: float,
                 next_weight: Optional[torch.Tensor] = None, next_out: Optional[torch.Tensor] = None) -> None:
     """x += rms(src) with ``weight``; with ``next_weight``, ``next_out = rms(x)`` of the new x in the same pass
-    (the norm behind a part, the residual addition and the norm in front of the next part)."""
+    (the norm behind a part, the residual addition and the norm in front of the next part); with ``next_out`` alone,
+    the new x itself in ``next_out``'s dtype (the next part reads the stream without a norm)."""
     _dev(src, weight, x, next_weight, next_out)
     _need(src.dtype == torch.float32 and x.dtype == torch.float32 and src.is_contiguous() and x.is_contiguous()
           and src.dim() == 2 and src.shape == x.shape, "rmsnorm_add: src and x must be contiguous float32 of one shape")
     R, E = x.shape
     _need(weight.numel() == E and weight.is_contiguous(), "rmsnorm_add: the gain's length differs from E")
-    _need((next_weight is None) == (next_out is None), "rmsnorm_add: the second norm needs its gain and its output")
+    _need(next_weight is None or next_out is not None, "rmsnorm_add: the second norm needs its output")
     if next_out is not None:
-        _need(next_weight.numel() == E and next_weight.is_contiguous() and next_out.is_contiguous()
+        _need((next_weight is None or (next_weight.numel() == E and next_weight.is_contiguous())) and next_out.is_contiguous()
               and tuple(next_out.shape) == (R, E), "rmsnorm_add: the second norm's operands differ from [R, E]")
     nb = R * E * 12 + _nbytes(weight, next_weight) + (0 if next_out is None else _nbytes(next_out))
     with _timed("rmsnorm_add", nb, 8 * R * E, "fp32"):

@@ -10,6 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import StepContext, build_feed_forward, build_mixer, build_norm, to_vector
+from .norms import STREAM_ITSELF
 
 
 class Block:
@@ -96,7 +97,9 @@ class Block:
                           lambda h, into: self.mixer.forward(ctx, h, into, call),
                           None if fused is None else (lambda norm, into: fused(ctx, norm, x, call) if into is None
                                                       else fused(ctx, norm, x, call, into=into)), part=self.mixer,
-                          scale=self.mixer_scale, next_pre=None if self.feed_forward is None or ctx.debug_hook is not None else self.pre_ff_norm)
+                          scale=self.mixer_scale,
+                          next_pre=None if self.feed_forward is None or ctx.debug_hook is not None else
+                          (self.pre_ff_norm if self.pre_ff_norm is not None else STREAM_ITSELF))
         if ctx.debug_hook is not None:
             ctx.emit(call.layer, "post_attention_residual", x)
         if self.feed_forward is not None:

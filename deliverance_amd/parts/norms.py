@@ -33,6 +33,10 @@ class LayerNorm(Norm):
 register_norm("layernorm", LayerNorm)
 
 
+# Handed to ``add_into`` in place of the next part's norm when that part has none in front of it.
+STREAM_ITSELF = object()
+
+
 class RmsNorm(Norm):
     """The row divided by its root mean square (eps inside the root), times ``gain_offset + weight``; all in
     32-bit.  Behind a part it can do three things in one pass over the row (``add_into``): normalise the
@@ -73,6 +77,10 @@ class RmsNorm(Norm):
                  next_name: str = "norm") -> Optional[torch.Tensor]:
         """x += norm(src).  With ``next_norm`` (an RMS norm of the same eps and offset) also returns
         ``next_norm(x)`` of the new x in the compute dtype; returns None when it did not do that."""
+        if next_norm is STREAM_ITSELF:             # the next part reads the stream without a norm: its copy, converted
+            h = ctx.buf(next_name, x.shape[0], self.width, ctx.dtype)
+            ops.rmsnorm_add(src, self.weight, x, self.gain_offset, self.eps, None, h)
+            return h
         nxt = next_norm if (type(next_norm) is RmsNorm and next_norm.eps == self.eps
                             and next_norm.gain_offset == self.gain_offset and next_norm.width == self.width) else None
         if nxt is None:
