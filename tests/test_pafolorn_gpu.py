@@ -418,6 +418,9 @@ def test_window_attention_kernel_against_sums_written_out(H, G, D, Dv, window, k
     scale = 0.7 / np.sqrt(D)
     decode = [(1, 0), (1, 37), (1, 500), (1, window + keep if window else 64)]
     portions = [(2, 0), (33, 5), (64, 130), (65, 0), (300, 200), (31, 470)]
+    if helpers.SIMT:                                   # (the simulated kernels: the same forms, fewer keys)
+        decode = [(1, 0), (1, 37), (1, window + keep + 9 if window else 64)]
+        portions = [(2, 0), (33, 5), (40, 130), (65, 0), (31, 170)]
     n_pages = sum(-(-(T + past) // page) for T, past in decode + portions) + 1
     order = list(rng.permutation(n_pages - 1) + 1)                      # page 0 belongs to nobody and holds NaN
     elems = G * page * (D + Dv)
