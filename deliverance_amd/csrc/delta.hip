@@ -12,8 +12,9 @@
 // neighbouring lanes, each with RPL consecutive rows in registers; the two sums over rows are taken inside the
 // lane and then over the 16 lanes by DPP additions.  A wavefront holds 4 columns, a workgroup's 4 walking wavefronts 16;
 // the grid is (sequences x heads x column blocks), each walking its sequence's portion in order; the tokens' numbers
-// come through LDS in blocks (see the kernel).  The order of every sum depends on D only, so a token's result
-// does not depend on how the sequence was cut into steps or on its neighbours in the batch.
+// come through LDS in blocks (see the kernel).  The order of every sum depends on D and on the token's place among
+// its portion's groups of four, so a token's result does not depend on its neighbours in the batch, and on how the
+// sequence was cut into steps by 32-bit rounding only.
 //
 // A request's state row holds S as [H][Dv][D] (a column's rows side by side) at its start; a sequence without a
 // slot (a padding row of a fixed-shape step) starts from zeros and keeps nothing.
