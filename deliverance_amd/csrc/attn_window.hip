@@ -12,7 +12,8 @@
 // sum) are merged in LDS in the order of the phases.  A wavefront's tiles are the ones that hold kept first keys
 // below its window, then the window's; a row's sums run over its tiles in ascending order, so they depend on the
 // row's position, the window and KP only, never on how the prompt was cut or on the batch.  Decode rows take
-// RB = 1 (four phases share out the keys), portions up to 64 rows RB = 2, longer ones RB = 4.
+// RB = 1 (four phases share out the keys), portions up to 64 rows RB = 2, longer ones RB = 4, or fewer where 128 rows
+// a workgroup would leave compute units idle.
 //
 // Per tile, with MFMA 32x32x16 (the operand layouts of attn_prefill.hip):
 //   S^T[key, row] = K . Q^T      key rows straight from the pages, 16 bytes a lane and 16 dimensions
@@ -31,6 +32,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float aw_floatx16;
 
 #define AW_BK 32
 #define AW_WAVES 4
+#define AW_FEW_WORKGROUPS 1024    // 128-row workgroups below which smaller ones are ahead (see the launch)
 #define AW_LOG2E 1.4426950408889634f
 
 // D16: the key size rounded up, in sixteens; DT: 32-dimension tiles of the values
@@ -279,7 +281,13 @@ extern "C" int da_attn_window(const void* q, int q_ld, const void* cache, const 
   DA_REQUIRE(scale > 0.f, "attn_window: the score scale must be positive, found %g", (double)scale);
   DA_REQUIRE((long)n_seqs * Hq < (1L << 31) && max_query_len <= 65535 * 32, "attn_window: too many sequences, heads or rows for one launch");
   if (n_seqs == 0 || max_query_len == 0) return 0;
-  const int RB = max_query_len <= 32 ? 1 : (max_query_len <= 64 ? 2 : 4);
+  // Row blocks a workgroup by the longest portion; where that leaves few workgroups (a long prompt or two, few
+  // heads), smaller workgroups whose wavefronts also share out the keys.  The step's shape only.  Measured on MI355X,
+  // head size 64, a window of 512 keeping 4, microseconds with 128 / 64 / 32 rows a workgroup: 2 x 1,024 rows, 6 heads
+  // 70 / - / 26.5; 8 heads - / 34.4 / 27.3; 4,096 rows, 16 heads 77.3 / 76.6 / -; 8 x 1,024 rows, 16 heads 113 / - / -.
+  int RB = max_query_len <= 32 ? 1 : (max_query_len <= 64 ? 2 : 4);
+  const long wg4 = (long)Hq * n_seqs * da_ceil_div(max_query_len, 128);
+  if (RB == 4 && wg4 < AW_FEW_WORKGROUPS) RB = 2 * wg4 < AW_FEW_WORKGROUPS ? 1 : 2;
   const dim3 grid((unsigned)(Hq * n_seqs), (unsigned)da_ceil_div(max_query_len, 32 * RB)), block(AW_WAVES * DA_WAVE);
 #define AW_GO(N, M)                                                                                                  \
   hipLaunchKernelGGL((attn_window_kernel<N, M>), grid, block, 0, (hipStream_t)stream, (const bf16_t*)q, q_ld,        \
