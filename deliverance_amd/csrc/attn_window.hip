@@ -267,12 +267,13 @@ extern "C" int da_attn_window_takes(int D, int Dv, int page) {
 }
 
 // Sequences seq0 .. seq0 + n_seqs - 1 of the step; rows of sequence s are q_start[s] .. q_start[s + 1] - 1, the
-// last of them at position seq_lens[s] - 1.
+// last of them at position seq_lens[s] - 1.  form: 0, or the row blocks a workgroup (1, 2, 4).
 extern "C" int da_attn_window(const void* q, int q_ld, const void* cache, const int* block_table, int max_blocks,
                               const int* q_start, const int* seq_lens, int seq0, int n_seqs, int max_query_len, int Hq,
                               int Hkv, int D, int Dv, int page, float scale, int window, int keep_first, float softcap,
-                              void* out, int out_ld, void* stream) {
+                              void* out, int out_ld, int form, void* stream) {
   DA_REQUIRE(n_seqs >= 0 && Hq > 0 && Hkv > 0 && max_query_len >= 0, "attn_window: bad sizes");
+  DA_REQUIRE(form == 0 || form == 1 || form == 2 || form == 4, "attn_window: form %d (0 leaves the choice to the rule; 1, 2 or 4 row blocks)", form);
   DA_REQUIRE(Hq % Hkv == 0, "attn_window: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   DA_REQUIRE(da_attn_window_takes(D, Dv, page), "attn_window: head sizes %d and %d with pages of %d are not taken", D, Dv, page);
   DA_REQUIRE(q_ld >= Hq * D && q_ld % 8 == 0 && out_ld >= Hq * Dv, "attn_window: row lengths");
@@ -288,6 +289,7 @@ extern "C" int da_attn_window(const void* q, int q_ld, const void* cache, const 
   int RB = max_query_len <= 32 ? 1 : (max_query_len <= 64 ? 2 : 4);
   const long wg4 = (long)Hq * n_seqs * da_ceil_div(max_query_len, 128);
   if (RB == 4 && wg4 < AW_FEW_WORKGROUPS) RB = 2 * wg4 < AW_FEW_WORKGROUPS ? 1 : 2;
+  if (form) RB = form;                                   // (tests walk every form at small sizes)
   const dim3 grid((unsigned)(Hq * n_seqs), (unsigned)da_ceil_div(max_query_len, 32 * RB)), block(AW_WAVES * DA_WAVE);
 #define AW_GO(N, M)                                                                                                  \
   hipLaunchKernelGGL((attn_window_kernel<N, M>), grid, block, 0, (hipStream_t)stream, (const bf16_t*)q, q_ld,        \

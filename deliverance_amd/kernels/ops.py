@@ -98,7 +98,7 @@ _ARGTYPES = {
     "da_rmsnorm": [_VP, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
     "da_rmsnorm_add": [_VP, _VP, _I, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
     "da_attn_rel_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _F, _I, _VP, _I, _VP],
-    "da_attn_window": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _VP, _I, _VP],
+    "da_attn_window": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _VP, _I, _I, _VP],
     "da_attn_window_takes": [_I, _I, _I],
     "da_attn_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _I, _VP, _VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _I, _VP],
     "da_delta_rule": [_VP, _I, _I, _I, _I, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I,
@@ -1003,9 +1003,10 @@ def attention_prefill_rel(q: torch.Tensor, cache_slot: torch.Tensor, block_table
 def attention_window(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, q_start: torch.Tensor,
                      seq_lens: torch.Tensor, seq0: int, n_seqs: int, max_query_len: int, n_heads: int, n_kv_heads: int,
                      head_dim: int, v_head_dim: int, page: int, scale: float, window: Optional[int], keep_first: int,
-                     softcap: float, out: torch.Tensor) -> torch.Tensor:
+                     softcap: float, out: torch.Tensor, form: int = 0) -> torch.Tensor:
     """Attention of the sequences ``seq0 .. seq0 + n_seqs - 1`` of a step on the matrix cores, in bfloat16, with keys and
-    values of their own sizes, a cap on the scores and, with a window, ``keep_first`` first keys that stay visible."""
+    values of their own sizes, a cap on the scores and, with a window, ``keep_first`` first keys that stay visible.
+    ``form``: 0 leaves the workgroup's row blocks to the kernel's rule; 1, 2 or 4 fixes them."""
     _dev(q, cache_slot, block_table, q_start, seq_lens, out)
     _rows_2d(q, "q"); _rows_2d(out, "out")
     _need(q.dtype == cache_slot.dtype == out.dtype == torch.bfloat16, "attention_window: q, cache and out must be bfloat16")
@@ -1020,7 +1021,7 @@ def attention_window(q: torch.Tensor, cache_slot: torch.Tensor, block_table: tor
     _check(_lib().da_attn_window(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table), block_table.shape[1],
                                  _ptr(q_start), _ptr(seq_lens), seq0, n_seqs, max_query_len, n_heads, n_kv_heads, head_dim,
                                  v_head_dim, page, float(scale), int(window or 0), int(keep_first if window else 0),
-                                 float(softcap), _ptr(out), out.stride(0), _stream()))
+                                 float(softcap), _ptr(out), out.stride(0), int(form), _stream()))
     return out
 
 

@@ -466,11 +466,14 @@ def test_window_attention_kernel_against_sums_written_out(H, G, D, Dv, window, k
     cache_t, bt = dev(cache, torch.bfloat16), dev(np.stack(tables))
     nd = len(decode)
     ops.attention_window(q_all, cache_t, bt, dev(starts), dev(lens), 0, nd, 1, H, G, D, Dv, page, scale, window, keep, cap, out)
-    ops.attention_window(q_all, cache_t, bt, dev(starts), dev(lens), nd, len(portions), max(T for T, _ in portions), H, G, D, Dv,
-                         page, scale, window, keep, cap, out)
-    got, want = host(out), np.concatenate(wants)
-    assert np.isfinite(got).all()
-    assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max()
+    want = np.concatenate(wants)
+    for form in (0, 4, 2, 1):                              # the rule's choice, then every number of row blocks
+        out[starts[nd]:] = float("nan")
+        ops.attention_window(q_all, cache_t, bt, dev(starts), dev(lens), nd, len(portions), max(T for T, _ in portions), H, G, D,
+                             Dv, page, scale, window, keep, cap, out, form=form)
+        got = host(out)
+        assert np.isfinite(got).all(), form
+        assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max(), form
 
 
 # ------------------------------------------------------------------------------------------ parallel mixers, layer scale
