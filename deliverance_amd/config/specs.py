@@ -98,6 +98,14 @@ class AttentionSpec:
     qk_norm: Optional["QKNormSpec"] = None   # queries and keys normalised before any rotation
     score_softcap: float = 0.0               # positive: score <- cap * tanh(score / cap), after the scale
     keep_first: int = 0                      # with a window: the first keys of a sequence stay visible for good
+    # the values are the keys as projected, before any rotation: there is no value matrix (v_head_dim = head_dim)
+    values_are_keys: bool = False
+    # one more term in the softmax's denominator that has no value: None, "zero" (exp(0) = 1) or "learned"
+    # (exp(sink_h), a parameter ``sink`` per query head; not multiplied by the scale)
+    sink: Optional[str] = None
+    # the heads' results are multiplied, element by element, with this function of one more projection of the
+    # mixer's input before the output projection: None or "sigmoid" (parameter ``gate_weight`` [heads * value size, width])
+    out_gate: Optional[str] = None
 
     @property
     def value_dim(self) -> int:
@@ -105,14 +113,29 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class RampedSpeedsSpec:
+    """Slower turns for long contexts.  With place(t) = dims * ln(original / (2 pi t)) / (2 ln base),
+    lo = max(floor(place(fast)), 0) and hi = min(ceil(place(slow)), dims - 1), pair i keeps its speed where
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1) is 0 and turns ``factor`` times slower where it is 1:
+    speed_i <- speed_i / factor * ramp_i + speed_i * (1 - ramp_i).  Sine and cosine are multiplied by
+    0.1 ln(factor) + 1."""
+    factor: float
+    original: float
+    fast: float
+    slow: float
+
+
+@dataclass(frozen=True)
 class RotarySpec:
     """Pairs of the first ``dims`` entries of a query or key vector are turned by the angle position * speed_i,
     speed_i = base^(-2i / dims), i = 0 .. dims / 2 - 1; entries behind ``dims`` pass.  ``interleaved``: pair i is
-    (2i, 2i + 1), else (i, i + dims / 2).  (u, v) becomes (u cos a - v sin a, v cos a + u sin a)."""
+    (2i, 2i + 1), else (i, i + dims / 2).  (u, v) becomes (u cos a - v sin a, v cos a + u sin a).  ``scaling``
+    changes the speeds and the length of the turned pairs (``RampedSpeedsSpec``)."""
     kind: str            # "rotary"
     dims: int
     base: float
     interleaved: bool = True
+    scaling: Optional[RampedSpeedsSpec] = None
 
 
 @dataclass(frozen=True)
@@ -136,6 +159,27 @@ class LatentAttentionSpec:
     norm_eps: float
     rotary: RotarySpec
     window: Optional[int] = None
+    # a learned number per head (parameter ``sink``) whose exponential joins the softmax's denominator: it has no
+    # key and no value and is not multiplied by the scale
+    sink: bool = False
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with a fixed decay per head and neither softmax nor denominator.  Per head a matrix S
+    (``head_dim`` x ``v_head_dim``, 32-bit) is carried from token to token: S <- decay_h S + k v^T, o = S^T q.
+    q and k are turned by the position (``rotary``) and k is then multiplied by head_dim^-1/2.  Each head's o is
+    divided by its root mean square (``norm_eps``, no gain), the heads are multiplied by ``gate`` ("silu") of one
+    more projection and projected back to the width."""
+    kind: str            # "retention"
+    width: int
+    n_heads: int
+    head_dim: int
+    v_head_dim: int
+    decay: Tuple[float, ...]
+    norm_eps: float
+    rotary: Optional[RotarySpec] = None
+    gate: str = "silu"
 
 
 @dataclass(frozen=True)
@@ -200,11 +244,13 @@ class DenseFeedForwardSpec:
 
 @dataclass(frozen=True)
 class GatedFeedForwardSpec:
-    """``down(act(gate h) * (up h))``, no biases."""
+    """``down(act(gate h) * (up h))``, no biases.  The activation "glu_capped" takes ``limit``: with
+    g = min(gate h, limit) and u = clamp(up h, -limit, limit) the middle is g * logistic(1.702 g) * (u + 1)."""
     kind: str            # "gated"
     width: int
     inner: int
     activation: str
+    limit: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -215,8 +261,11 @@ class ExpertsFeedForwardSpec:
     [n_experts, width] gives 32-bit logits z; the ``top`` experts with the largest logistic(z) are used, with those
     scores as weights (``renormalize``: divided by their sum).  ``gated``: an expert is down(act(gate h) * (up h)),
     else down(act(up h)).  ``weight_on``: "output" (weight * expert(h)) or "input" (expert(weight * h)).
-    ``shared_inner`` > 0: one more feed-forward of that many columns, of the ungated form, runs for every token
-    with weight 1 and is added."""
+    ``router == "softmax_top"``: logits z = matrix h + bias (32-bit); the ``top`` largest logits are used (the lower
+    index wins a tie), with the softmax over just those as weights.
+    ``shared_inner`` > 0: one more feed-forward of that many columns runs for every token with weight 1 and is
+    added; it is ungated, or (``shared_gated``) of the gated form with ``shared_limit``.  ``limit``: the constant of
+    the activation "glu_capped" (``GatedFeedForwardSpec``)."""
     kind: str            # "experts"
     width: int
     inner: int
@@ -230,6 +279,10 @@ class ExpertsFeedForwardSpec:
     renormalize: bool = False
     shared_inner: int = 0
     shared_activation: Optional[str] = None
+    limit: float = 0.0
+    shared_gated: bool = False
+    shared_limit: float = 0.0
+    router_bias: bool = False
 
 
 @dataclass(frozen=True)
@@ -264,11 +317,13 @@ class LayerCall:
 
     ``layer`` indexes ``ModelConfig.layers`` (a layer may be named twice), ``cache`` is
     the cache slot its mixer uses, and ``write`` is False when the mixer only reads a
-    slot that another call has filled in the same step.
+    slot that another call has filled in the same step.  ``mix_input``: right before this
+    call the stream becomes W [stream; embedding output] (``ModelConfig.input_mix``).
     """
     layer: int
     cache: int
     write: bool = True
+    mix_input: bool = False
 
 
 @dataclass(frozen=True)
@@ -293,6 +348,9 @@ class ModelConfig:
     logit_softcap: float = 0.0
     # a norm on the embedded tokens before the first layer (parameters "embed_norm")
     embed_norm: Optional[NormSpec] = None
+    # a matrix [width, 2 width] (parameter "input_mix") that run-order entries with ``mix_input`` apply to the
+    # stream beside the embedding output (the stream's half first)
+    input_mix: bool = False
 
     @property
     def n_cache_slots(self) -> int:

@@ -23,15 +23,15 @@ template <typename T>
 __global__ void __launch_bounds__(128)
 rotary_kernel(const T* __restrict__ src, int src_ld, int src_hs, T* __restrict__ dst, int dst_ld, int dst_hs,
               const int* __restrict__ positions, const double* __restrict__ speeds, int H, int width, int dims,
-              int interleaved) {
+              int interleaved, float mag) {
   __shared__ float cs[ROT_MAX_HALF], sn[ROT_MAX_HALF];
   const int n = blockIdx.x, half = dims / 2;
   const double p = (double)positions[n];
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     double s, c;
     sincos(p * speeds[i], &s, &c);
-    cs[i] = (float)c;
-    sn[i] = (float)s;
+    cs[i] = (float)c * mag;                             // (mag: the length that a turned pair gains; 1 as a rule)
+    sn[i] = (float)s * mag;
   }
   __syncthreads();
   const T* in = src + (size_t)n * src_ld;
@@ -57,7 +57,7 @@ rotary_kernel(const T* __restrict__ src, int src_ld, int src_hs, T* __restrict__
 
 extern "C" int da_rotary(const void* src, int src_ld, int src_hs, void* dst, int dst_ld, int dst_hs, int dtype,
                          const int* positions, const double* speeds, int N, int H, int width, int dims, int interleaved,
-                         void* stream) {
+                         float mag, void* stream) {
   DA_REQUIRE(N >= 0 && H > 0 && width > 0 && dims >= 0 && dims <= width && dims % 2 == 0, "rotary: bad sizes");
   DA_REQUIRE(dims / 2 <= ROT_MAX_HALF, "rotary: %d turned entries, %d are taken", dims, 2 * ROT_MAX_HALF);
   DA_REQUIRE(src_ld >= (H - 1) * src_hs + width && dst_ld >= (H - 1) * dst_hs + width && src_hs >= width && dst_hs >= width,
@@ -65,10 +65,10 @@ extern "C" int da_rotary(const void* src, int src_ld, int src_hs, void* dst, int
   if (N == 0) return 0;
   if (dtype == DA_BF16)
     hipLaunchKernelGGL(rotary_kernel<bf16_t>, dim3(N), dim3(128), 0, (hipStream_t)stream, (const bf16_t*)src, src_ld, src_hs,
-                       (bf16_t*)dst, dst_ld, dst_hs, positions, speeds, H, width, dims, interleaved);
+                       (bf16_t*)dst, dst_ld, dst_hs, positions, speeds, H, width, dims, interleaved, mag);
   else
     hipLaunchKernelGGL(rotary_kernel<float>, dim3(N), dim3(128), 0, (hipStream_t)stream, (const float*)src, src_ld, src_hs,
-                       (float*)dst, dst_ld, dst_hs, positions, speeds, H, width, dims, interleaved);
+                       (float*)dst, dst_ld, dst_hs, positions, speeds, H, width, dims, interleaved, mag);
   DA_CHECK_LAUNCH("rotary");
   return 0;
 }
@@ -80,8 +80,8 @@ __global__ void __launch_bounds__(128)
 latent_prepare_kernel(const TIN* __restrict__ down, int ld, int Rq, int R, int Dr, const void* __restrict__ gq,
                       int gq_dtype, const void* __restrict__ gc, int gc_dtype, float eps,
                       const int* __restrict__ positions, const int* __restrict__ slot_map,
-                      const double* __restrict__ speeds, int dims, int interleaved, TOUT* __restrict__ cq, int cq_ld,
-                      TOUT* __restrict__ cache, int page) {
+                      const double* __restrict__ speeds, int dims, int interleaved, float mag, TOUT* __restrict__ cq,
+                      int cq_ld, TOUT* __restrict__ cache, int page) {
   const int n = blockIdx.x, lane = threadIdx.x % DA_WAVE, wave = threadIdx.x / DA_WAVE;
   const TIN* row = down + (size_t)n * ld;
   if (wave == 0) {
@@ -116,7 +116,8 @@ latent_prepare_kernel(const TIN* __restrict__ down, int ld, int Rq, int R, int D
       double s, co;
       sincos(p * speeds[i], &s, &co);
       const float a = to_f32(kr[d]), b = to_f32(kr[other]);
-      r = first ? a * (float)co - b * (float)s : a * (float)co + b * (float)s;
+      const float cf = (float)co * mag, sf = (float)s * mag;
+      r = first ? a * cf - b * sf : a * cf + b * sf;
     }
     from_f32(&dst[R + d], r);
   }
@@ -124,8 +125,8 @@ latent_prepare_kernel(const TIN* __restrict__ down, int ld, int Rq, int R, int D
 
 extern "C" int da_latent_prepare(const void* down, int in_dtype, int ld, int Rq, int R, int Dr, const void* gq, int gq_dtype,
                                  const void* gc, int gc_dtype, float eps, const int* positions, const int* slot_map,
-                                 const double* speeds, int dims, int interleaved, void* cq, int cq_ld, void* cache,
-                                 int out_dtype, int page, int N, void* stream) {
+                                 const double* speeds, int dims, int interleaved, float mag, void* cq, int cq_ld,
+                                 void* cache, int out_dtype, int page, int N, void* stream) {
   DA_REQUIRE(N >= 0 && Rq >= 0 && R > 0 && Dr >= 0 && ld >= Rq + R + Dr && page > 0, "latent_prepare: bad sizes");
   DA_REQUIRE(dims >= 0 && dims <= Dr && dims % 2 == 0, "latent_prepare: %d turned entries of %d", dims, Dr);
   DA_REQUIRE(Rq == 0 || (cq != nullptr && cq_ld >= Rq && gq != nullptr), "latent_prepare: the query latent needs a gain and a place");
@@ -133,7 +134,7 @@ extern "C" int da_latent_prepare(const void* down, int in_dtype, int ld, int Rq,
   if (N == 0) return 0;
 #define DA_LP_GO(TIN, TOUT)                                                                                              \
   hipLaunchKernelGGL((latent_prepare_kernel<TIN, TOUT>), dim3(N), dim3(128), 0, (hipStream_t)stream, (const TIN*)down, ld, \
-                     Rq, R, Dr, gq, gq_dtype, gc, gc_dtype, eps, positions, slot_map, speeds, dims, interleaved,          \
+                     Rq, R, Dr, gq, gq_dtype, gc, gc_dtype, eps, positions, slot_map, speeds, dims, interleaved, mag,     \
                      (TOUT*)cq, cq_ld, (TOUT*)cache, page)
   if (in_dtype == DA_F32 && out_dtype == DA_F32) DA_LP_GO(float, float);
   else if (in_dtype == DA_F32) DA_LP_GO(float, bf16_t);
@@ -146,12 +147,14 @@ extern "C" int da_latent_prepare(const void* down, int in_dtype, int ld, int Rq,
 
 // For the token at position p, head h, rows j in [lo, p] of its sequence:
 //   s_j = (q'[n, h, :] . row_j) * scale,  w = softmax(s),  o[n, h, :] = sum_j w_j row_j[0 .. Dv)        (32-bit)
+// With `sink` ([Hq], 32-bit) the softmax's denominator also holds exp(sink[h]): no key, no value, not scaled.
 // Rows are walked in chunks of 64 from lo, so the order of the sums depends on the token's position only.
 template <typename T>
 __global__ void __launch_bounds__(DA_WAVE)
 attn_latent_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cache, const int* __restrict__ block_table,
                        int max_blocks, const int* __restrict__ seq_of_token, const int* __restrict__ positions, int Hq,
-                       int D, int Dv, int page, float scale, int window, T* __restrict__ out, int out_ld) {
+                       int D, int Dv, int page, float scale, int window, const float* __restrict__ sink,
+                       T* __restrict__ out, int out_ld) {
   __shared__ float qs[LAT_MAX_D];
   __shared__ float ps[DA_WAVE];
   __shared__ long long roff[DA_WAVE];
@@ -200,7 +203,14 @@ attn_latent_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ 
     }
     __syncthreads();
   }
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  float shrink = 1.f;
+  if (sink) {
+    const float s0 = sink[h];
+    const float m_all = fmaxf(m, s0);
+    shrink = m == -INFINITY ? 0.f : expf(m - m_all);
+    l = l * shrink + expf(s0 - m_all);
+  }
+  const float inv = l > 0.f ? shrink / l : 0.f;
 #pragma unroll
   for (int i = 0; i < LAT_MAX_D / DA_WAVE; ++i) {
     const int d = lane + i * DA_WAVE;
@@ -210,7 +220,8 @@ attn_latent_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ 
 
 extern "C" int da_attn_latent_ref(const void* q, int q_ld, const void* cache, int dtype, const int* block_table,
                                   int max_blocks, const int* seq_of_token, const int* positions, int N, int Hq, int D,
-                                  int Dv, int page, float scale, int window, void* out, int out_ld, void* stream) {
+                                  int Dv, int page, float scale, int window, const float* sink, void* out, int out_ld,
+                                  void* stream) {
   DA_REQUIRE(N >= 0 && Hq > 0 && D > 0 && Dv > 0 && Dv <= D && page > 0, "attn_latent_ref: bad sizes");
   DA_REQUIRE(D <= LAT_MAX_D, "attn_latent_ref: rows of %d entries, %d are taken", D, LAT_MAX_D);
   DA_REQUIRE(q_ld >= Hq * D && out_ld >= Hq * Dv, "attn_latent_ref: row lengths too small");
@@ -219,11 +230,11 @@ extern "C" int da_attn_latent_ref(const void* q, int q_ld, const void* cache, in
   if (dtype == DA_BF16)
     hipLaunchKernelGGL(attn_latent_ref_kernel<bf16_t>, dim3(N * Hq), dim3(DA_WAVE), 0, (hipStream_t)stream, (const bf16_t*)q,
                        q_ld, (const bf16_t*)cache, block_table, max_blocks, seq_of_token, positions, Hq, D, Dv, page, scale,
-                       window, (bf16_t*)out, out_ld);
+                       window, sink, (bf16_t*)out, out_ld);
   else
     hipLaunchKernelGGL(attn_latent_ref_kernel<float>, dim3(N * Hq), dim3(DA_WAVE), 0, (hipStream_t)stream, (const float*)q,
                        q_ld, (const float*)cache, block_table, max_blocks, seq_of_token, positions, Hq, D, Dv, page, scale,
-                       window, (float*)out, out_ld);
+                       window, sink, (float*)out, out_ld);
   DA_CHECK_LAUNCH("attn_latent_ref");
   return 0;
 }

@@ -9,7 +9,8 @@
 // lane % 16.  The softmax runs over a wavefront's own 16 rows in 32-bit; the weights pass through LDS to become
 // the first operand of the second product.  The next tile's rows are asked for before this tile's arithmetic.
 // Tiles are walked from the first visible key in steps of 32, so the order of a row's sums depends on the row's
-// own sequence only.
+// own sequence only.  With `sink` ([H], 32-bit) the softmax's denominator also holds exp(sink[head]), which has no
+// key and no value and is not scaled; it joins once, where a row's result is final (here, or in the merge).
 #include "gemm_common.h"
 
 #define LM_ROWS 64            // query rows a workgroup
@@ -22,7 +23,8 @@ __global__ void __launch_bounds__(256)
 attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                         const int* __restrict__ block_table, int max_blocks, const int* __restrict__ q_start,
                         const int* __restrict__ seq_lens, int H, int D, int R, int page, float scale_log2e, int window,
-                        bf16_t* __restrict__ out, int out_ld, int seq0, int n_splits, float* __restrict__ partial) {
+                        bf16_t* __restrict__ out, int out_ld, int seq0, int n_splits, float* __restrict__ partial,
+                        const float* __restrict__ sink) {
   constexpr int D32 = DB * 32;
   constexpr int ldk = D32 + LM_PAD;                   // entries of a row of the key tile
   constexpr int ldv = LM_KEYS + LM_PAD;               // entries of a row of the value tile (one entry of R)
@@ -225,7 +227,14 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
   for (int r = 0; r < 4; ++r) {
     const int row = row0 + wave * 16 + 4 * fg + r;
     if (row >= T * H) continue;
-    const float inv = l[r] > 0.f ? 1.0f / l[r] : 0.f;
+    float shrink = 1.f, lr = l[r];
+    if (sink) {                                       // base-2 domain, as the maxima are
+      const float s0 = sink[row % H] * 1.4426950408889634f;
+      const float m_all = fmaxf(m[r], s0);
+      shrink = m[r] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[r] - m_all);
+      lr = lr * shrink + __builtin_amdgcn_exp2f(s0 - m_all);
+    }
+    const float inv = lr > 0.f ? shrink / lr : 0.f;
     bf16_t* op = out + (size_t)(first + row / H) * out_ld + (size_t)(row % H) * R;
 #pragma unroll
     for (int i = 0; i < RB; ++i)
@@ -237,7 +246,7 @@ attn_latent_mfma_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __
 #define LM_MAX_SPLITS 64
 __global__ void __launch_bounds__(128)
 attn_latent_merge_kernel(const float* __restrict__ partial, int rows_cap, int n_splits, const int* __restrict__ q_start,
-                         int seq0, int H, int R, bf16_t* __restrict__ out, int out_ld) {
+                         int seq0, int H, int R, bf16_t* __restrict__ out, int out_ld, const float* __restrict__ sink) {
   __shared__ float wz[LM_MAX_SPLITS];
   const int s_local = blockIdx.y, row = blockIdx.x;
   const int first = q_start[seq0 + s_local], T = q_start[seq0 + s_local + 1] - first;
@@ -247,9 +256,10 @@ attn_latent_merge_kernel(const float* __restrict__ partial, int rows_cap, int n_
     const int z = threadIdx.x;
     const float mz = z < n_splits ? pp[(size_t)z * (R + 2)] : -INFINITY;
     const float lz = z < n_splits ? pp[(size_t)z * (R + 2) + 1] : 0.f;
-    const float M = wave_max(mz);
+    const float s0 = sink ? sink[row % H] * 1.4426950408889634f : -INFINITY;
+    const float M = fmaxf(wave_max(mz), s0);
     const float e = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - M);
-    const float L = wave_sum(lz * e);
+    const float L = wave_sum(lz * e) + (sink ? __builtin_amdgcn_exp2f(s0 - M) : 0.f);
     if (z < n_splits) wz[z] = L > 0.f ? e / L : 0.f;
   }
   __syncthreads();
@@ -289,7 +299,7 @@ extern "C" long da_attn_latent_partial_floats(int S, int max_query_len, int H, i
 extern "C" int da_attn_latent_mfma(const void* q, int q_ld, const void* cache, const int* block_table, int max_blocks,
                                    const int* q_start, const int* seq_lens, int seq0, int S, int max_query_len, int H, int D,
                                    int R, int page, float scale, int window, void* out, int out_ld, int n_splits,
-                                   float* partial, long partial_floats, void* stream) {
+                                   float* partial, long partial_floats, const float* sink, void* stream) {
   DA_REQUIRE(S >= 0 && seq0 >= 0 && H > 0 && page > 0 && max_blocks > 0 && max_query_len > 0 && window >= 0 && n_splits >= 1,
              "attn_latent_mfma: bad sizes");
   DA_REQUIRE(da_attn_latent_mfma_takes(D, R), "attn_latent_mfma: rows of %d entries with %d of them values are not taken", D, R);
@@ -306,7 +316,7 @@ extern "C" int da_attn_latent_mfma(const void* q, int q_ld, const void* cache, c
 #define DA_LM_GO(DB, RB)                                                                                                  \
   hipLaunchKernelGGL((attn_latent_mfma_kernel<DB, RB>), grid, block, 0, st, (const bf16_t*)q, q_ld, (const bf16_t*)cache,   \
                      block_table, max_blocks, q_start, seq_lens, H, D, R, page, sl2, window, (bf16_t*)out, out_ld, seq0,   \
-                     n_splits, partial)
+                     n_splits, partial, sink)
   if (D <= 128 && R <= 128) DA_LM_GO(4, 8);
   else if (D <= 256 && R <= 256) DA_LM_GO(8, 16);
   else if (D <= 384 && R <= 384) DA_LM_GO(12, 24);
@@ -315,7 +325,7 @@ extern "C" int da_attn_latent_mfma(const void* q, int q_ld, const void* cache, c
   DA_CHECK_LAUNCH("attn_latent_mfma");
   if (n_splits > 1) {
     hipLaunchKernelGGL(attn_latent_merge_kernel, dim3(max_query_len * H, S), dim3(128), 0, st, partial, (int)grid.x * LM_ROWS,
-                       n_splits, q_start, seq0, H, R, (bf16_t*)out, out_ld);
+                       n_splits, q_start, seq0, H, R, (bf16_t*)out, out_ld, sink);
     DA_CHECK_LAUNCH("attn_latent_merge");
   }
   return 0;

@@ -9,6 +9,8 @@
 // With a window w the keys are j in [p - w + 1, p] and, with keep_first, also j < keep_first: the first keys of a
 // sequence stay visible at their true positions.
 //   w = softmax(s),  o = sum_j w_j v_j                                 (all in 32-bit)
+// `sink` (optional, [Hq], 32-bit): the softmax's denominator also holds exp(sink[h]), a term without a key or a
+// value that is not scaled.  `gate` (optional, rows like out): o <- o * logistic(gate).
 // `bias` (optional) is a table by distance, [Hq][n_dist], 32-bit: whoever owns the rule that turns a
 // distance into a learned value (buckets, slopes) writes it out once per layer up to the distance from
 // which it no longer changes.
@@ -28,6 +30,7 @@ attn_rel_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cac
                     const int* __restrict__ seq_of_token, const int* __restrict__ positions,
                     int Hq, int Hkv, int D, int Dv, int page, float scale, int window,
                     const float* __restrict__ bias, int n_dist, float t_coef, int t_every, float softcap, int keep_first,
+                    const float* __restrict__ sink, const T* __restrict__ gate, int gate_ld,
                     T* __restrict__ out, int out_ld) {
   __shared__ float qs[REL_MAX_D];
   __shared__ float ps[DA_WAVE];
@@ -97,19 +100,30 @@ attn_rel_ref_kernel(const T* __restrict__ q, int q_ld, const T* __restrict__ cac
     __syncthreads();
   }
   }
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  float shrink = 1.f;
+  if (sink) {                                            // one more term of the denominator, counted once
+    const float s0 = sink[h];
+    const float m_all = fmaxf(m, s0);
+    shrink = m == -INFINITY ? 0.f : expf(m - m_all);
+    l = l * shrink + expf(s0 - m_all);
+  }
+  const float inv = l > 0.f ? shrink / l : 0.f;
 #pragma unroll
   for (int i = 0; i < REL_MAX_D / DA_WAVE; ++i) {
     const int d = lane + i * DA_WAVE;
-    if (d < Dv) from_f32(&out[(size_t)n * out_ld + h * Dv + d], acc[i] * inv);
+    if (d < Dv) {
+      float r = acc[i] * inv;
+      if (gate) r *= 1.0f / (1.0f + expf(-to_f32(gate[(size_t)n * gate_ld + h * Dv + d])));
+      from_f32(&out[(size_t)n * out_ld + h * Dv + d], r);
+    }
   }
 }
 
 extern "C" int da_attn_rel_ref(const void* q, int q_ld, const void* cache, int dtype, const int* block_table,
                                int max_blocks, const int* seq_of_token, const int* positions, int N, int Hq, int Hkv,
                                int D, int Dv, int page, float scale, int window, const float* bias, int n_dist,
-                               float t_coef, int t_every, float softcap, int keep_first, void* out, int out_ld,
-                               void* stream) {
+                               float t_coef, int t_every, float softcap, int keep_first, const float* sink,
+                               const void* gate, int gate_ld, void* out, int out_ld, void* stream) {
   DA_REQUIRE(N >= 0 && Hq > 0 && Hkv > 0 && D > 0 && Dv > 0 && page > 0, "attn_rel_ref: bad sizes");
   DA_REQUIRE(Hq % Hkv == 0, "attn_rel_ref: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   DA_REQUIRE(D <= REL_MAX_D && Dv <= REL_MAX_D, "attn_rel_ref: head sizes %d, %d exceed %d", D, Dv, REL_MAX_D);
@@ -118,15 +132,18 @@ extern "C" int da_attn_rel_ref(const void* q, int q_ld, const void* cache, int d
   DA_REQUIRE(!bias || n_dist > 0, "attn_rel_ref: a bias table without entries");
   DA_REQUIRE(t_every >= 0, "attn_rel_ref: bad temperature period %d", t_every);
   DA_REQUIRE(softcap >= 0.f && keep_first >= 0, "attn_rel_ref: bad score cap or kept first keys");
+  DA_REQUIRE(!gate || gate_ld >= Hq * Dv, "attn_rel_ref: the gate's rows are too short");
   if (N == 0) return 0;
   if (dtype == DA_BF16)
     hipLaunchKernelGGL(attn_rel_ref_kernel<bf16_t>, dim3(N * Hq), dim3(DA_WAVE), 0, (hipStream_t)stream,
                        (const bf16_t*)q, q_ld, (const bf16_t*)cache, block_table, max_blocks, seq_of_token, positions,
-                       Hq, Hkv, D, Dv, page, scale, window, bias, n_dist, t_coef, t_every, softcap, keep_first, (bf16_t*)out, out_ld);
+                       Hq, Hkv, D, Dv, page, scale, window, bias, n_dist, t_coef, t_every, softcap, keep_first, sink,
+                       (const bf16_t*)gate, gate_ld, (bf16_t*)out, out_ld);
   else
     hipLaunchKernelGGL(attn_rel_ref_kernel<float>, dim3(N * Hq), dim3(DA_WAVE), 0, (hipStream_t)stream,
                        (const float*)q, q_ld, (const float*)cache, block_table, max_blocks, seq_of_token, positions,
-                       Hq, Hkv, D, Dv, page, scale, window, bias, n_dist, t_coef, t_every, softcap, keep_first, (float*)out, out_ld);
+                       Hq, Hkv, D, Dv, page, scale, window, bias, n_dist, t_coef, t_every, softcap, keep_first, sink,
+                       (const float*)gate, gate_ld, (float*)out, out_ld);
   DA_CHECK_LAUNCH("attn_rel_ref");
   return 0;
 }

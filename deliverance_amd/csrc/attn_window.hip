@@ -5,6 +5,9 @@
 // For the row at position p, key j is seen when j <= p and (no window, or p - j < window, or j < keep_first);
 //   s_j = cap((q . k_j) * scale),  cap(s) = softcap * tanh(s / softcap)   (s itself when softcap is 0)
 //   o   = sum_j softmax(s)_j v_j                                           (scores, weights and sums in 32-bit)
+// `sink` (optional, [Hq], 32-bit): the softmax's denominator also holds exp(sink[h]), a term without a key or a
+// value that is not scaled; it joins once, after the phases have been merged.  `gate` (optional, rows like out):
+// o <- o * logistic(gate), in the store.
 //
 // One workgroup of four wavefronts per (sequence, query head, 32 * RB rows).  A wavefront owns a row block of 32
 // rows and one of KP = 4 / RB key phases: keys come in aligned tiles of 32, tile a (keys 32 a ..) belongs to phase
@@ -47,7 +50,8 @@ __global__ void __launch_bounds__(AW_WAVES * DA_WAVE)
 attn_window_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restrict__ cache,
                    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ q_start,
                    const int* __restrict__ seq_lens, int seq0, int Hq, int Hkv, int D, int Dv, int page, float scale,
-                   int window, int keep_first, float softcap, bf16_t* __restrict__ out, int out_ld, int RB) {
+                   int window, int keep_first, float softcap, const float* __restrict__ sink,
+                   const bf16_t* __restrict__ gate, int gate_ld, bf16_t* __restrict__ out, int out_ld, int RB) {
   constexpr int PER = DT * 16 + 2;
   __shared__ float mg[3 * PER * DA_WAVE];              // (KP - 1) * RB <= 3 partial results
   const int KP = AW_WAVES / RB;
@@ -249,14 +253,32 @@ attn_window_kernel(const bf16_t* __restrict__ q, int q_ld, const bf16_t* __restr
     }
   }
   if (qi < T) {
-    const float inv = l > 0.f ? 1.0f / l : 0.f;          // a sequence of length 0 (padding) gives zeros
+    float shrink = 1.f;
+    if (sink) {                                          // the term without a key, in the base-2 domain
+      const float s0 = sink[h] * AW_LOG2E;
+      const float m_all = fmaxf(m, s0);
+      shrink = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m_all);
+      l = l * shrink + __builtin_amdgcn_exp2f(s0 - m_all);
+    }
+    const float inv = l > 0.f ? shrink / l : 0.f;        // a sequence of length 0 (padding) gives zeros
     bf16_t* orow = out + (size_t)(row0 + qi) * out_ld + h * Dv;
+    const bf16_t* grow = gate ? gate + (size_t)(row0 + qi) * gate_ld + h * Dv : nullptr;
 #pragma unroll
     for (int i = 0; i < DT; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int d = i * 32 + 8 * (r / 4) + 4 * hf + (r % 4);
-        if (d < Dv) orow[d] = f32_to_bf16(acc_o[i][r] * inv);
+      for (int r = 0; r < 16; r += 4) {
+        const int d = i * 32 + 8 * (r / 4) + 4 * hf;     // four neighbouring entries
+        if (d < Dv) {
+          float g4[4] = {1.f, 1.f, 1.f, 1.f};
+          if (grow) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (d + e < Dv) g4[e] = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-AW_LOG2E * bf16_to_f32(grow[d + e])));
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (d + e < Dv) orow[d + e] = f32_to_bf16(acc_o[i][r + e] * inv * g4[e]);
+        }
       }
   }
 }
@@ -271,7 +293,8 @@ extern "C" int da_attn_window_takes(int D, int Dv, int page) {
 extern "C" int da_attn_window(const void* q, int q_ld, const void* cache, const int* block_table, int max_blocks,
                               const int* q_start, const int* seq_lens, int seq0, int n_seqs, int max_query_len, int Hq,
                               int Hkv, int D, int Dv, int page, float scale, int window, int keep_first, float softcap,
-                              void* out, int out_ld, int form, void* stream) {
+                              const float* sink, const void* gate, int gate_ld, void* out, int out_ld, int form,
+                              void* stream) {
   DA_REQUIRE(n_seqs >= 0 && Hq > 0 && Hkv > 0 && max_query_len >= 0, "attn_window: bad sizes");
   DA_REQUIRE(form == 0 || form == 1 || form == 2 || form == 4, "attn_window: form %d (0 leaves the choice to the rule; 1, 2 or 4 row blocks)", form);
   DA_REQUIRE(Hq % Hkv == 0, "attn_window: %d query heads are not a multiple of %d key heads", Hq, Hkv);
@@ -280,6 +303,7 @@ extern "C" int da_attn_window(const void* q, int q_ld, const void* cache, const 
   DA_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)cache % 16 == 0), "attn_window: operands must be 16-byte aligned");
   DA_REQUIRE(window >= 0 && keep_first >= 0 && softcap >= 0.f && max_blocks > 0, "attn_window: bad window, kept keys, cap or block table");
   DA_REQUIRE(scale > 0.f, "attn_window: the score scale must be positive, found %g", (double)scale);
+  DA_REQUIRE(!gate || gate_ld >= Hq * Dv, "attn_window: the gate's rows are too short");
   DA_REQUIRE((long)n_seqs * Hq < (1L << 31) && max_query_len <= 65535 * 32, "attn_window: too many sequences, heads or rows for one launch");
   if (n_seqs == 0 || max_query_len == 0) return 0;
   // Row blocks a workgroup by the longest portion; where that leaves few workgroups (a long prompt or two, few
@@ -294,7 +318,7 @@ extern "C" int da_attn_window(const void* q, int q_ld, const void* cache, const 
 #define AW_GO(N, M)                                                                                                  \
   hipLaunchKernelGGL((attn_window_kernel<N, M>), grid, block, 0, (hipStream_t)stream, (const bf16_t*)q, q_ld,        \
                      (const bf16_t*)cache, block_table, max_blocks, q_start, seq_lens, seq0, Hq, Hkv, D, Dv, page,   \
-                     scale, window, keep_first, softcap, (bf16_t*)out, out_ld, RB)
+                     scale, window, keep_first, softcap, sink, (const bf16_t*)gate, gate_ld, (bf16_t*)out, out_ld, RB)
 #define AW_VALUES(N)                 \
   do {                               \
     if (Dv <= 32) AW_GO(N, 1);       \

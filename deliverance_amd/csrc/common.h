@@ -17,7 +17,10 @@
 #define DA_ACT_RELU 3
 #define DA_ACT_SILU 4
 #define DA_ACT_RELU2 5      // the square of max(x, 0)
-#define DA_ACT_LAST DA_ACT_RELU2
+// Only as the activation of a gated pair (gated_mid below): with g = min(gate, limit) and u = clamp(up, -limit,
+// limit) the middle is g * logistic(1.702 g) * (u + 1).
+#define DA_ACT_GLU_CAPPED 6
+#define DA_ACT_LAST DA_ACT_GLU_CAPPED
 
 #define DA_WAVE 64
 
@@ -228,6 +231,20 @@ __device__ __forceinline__ float apply_act_bf16(float x, int act) {
   }
   if (act == DA_ACT_SILU) return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * x));
   return apply_act(x, act);
+}
+
+// The middle of a gated feed-forward from the two products' sums: act(g) * u, or the capped form with its limit.
+// FAST: where the result is rounded to bfloat16 anyway (the hardware's exp2 and reciprocal).
+template <bool FAST>
+__device__ __forceinline__ float gated_mid(float g, float u, int act, float limit) {
+  if (act == DA_ACT_GLU_CAPPED) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    const float sg = FAST ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.702f * 1.4426950408889634f * g))
+                          : 1.0f / (1.0f + expf(-1.702f * g));
+    return g * sg * (u + 1.0f);
+  }
+  return (FAST ? apply_act_bf16(g, act) : apply_act(g, act)) * u;
 }
 
 static inline int da_ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

@@ -98,7 +98,7 @@ template <typename T, int MODE>
 __global__ void __launch_bounds__(256)
 moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
                        const int* __restrict__ tile_expert, const T* __restrict__ w, void* __restrict__ out, int ldo,
-                       int K, int F, int act, const float* __restrict__ slot_scale) {
+                       int K, int F, int act, const float* __restrict__ slot_scale, float limit) {
   constexpr bool GATED = MODE == MOE_GATED, GATHER = MODE != MOE_DOWN;
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
@@ -179,10 +179,7 @@ moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__
       if (n >= F) continue;
       const size_t o = (size_t)(m0 + r) * ldo + n;
       if (GATED) {
-        if (DTypeOf<T>::value == DA_BF16)
-          from_f32(&((T*)out)[o], apply_act_bf16(sc * acc[0][i][j], act) * (sc * acc[1][i][j]));
-        else
-          from_f32(&((T*)out)[o], apply_act(sc * acc[0][i][j], act) * (sc * acc[1][i][j]));
+        from_f32(&((T*)out)[o], gated_mid<DTypeOf<T>::value == DA_BF16>(sc * acc[0][i][j], sc * acc[1][i][j], act, limit));
       } else if (MODE == MOE_UP) {
         from_f32(&((T*)out)[o], DTypeOf<T>::value == DA_BF16 ? apply_act_bf16(sc * acc[0][i][j], act) : apply_act(sc * acc[0][i][j], act));
       } else {
@@ -193,17 +190,19 @@ moe_product_ref_kernel(const T* __restrict__ a, int lda, const int* __restrict__
 }
 
 extern "C" int da_moe_gated_ref(const void* a, int lda, int dtype, const int* row_of_slot, const int* tile_expert,
-                                const void* w, void* mid, int ldm, int T_cap, int K, int F, int act, void* stream) {
+                                const void* w, void* mid, int ldm, int T_cap, int K, int F, int act, float limit,
+                                void* stream) {
   DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_gated_ref: bad sizes");
+  DA_REQUIRE(act != DA_ACT_GLU_CAPPED || limit > 0.f, "moe_gated_ref: the capped form needs a positive limit");
   DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "moe_gated_ref: unknown activation %d", act);
   if (T_cap == 0) return 0;
   dim3 grid(da_ceil_div(F, MT), T_cap);
   if (dtype == DA_BF16)
     hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, MOE_GATED>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a,
-                       lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, nullptr);
+                       lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, nullptr, limit);
   else
     hipLaunchKernelGGL((moe_product_ref_kernel<float, MOE_GATED>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)a,
-                       lda, row_of_slot, tile_expert, (const float*)w, mid, ldm, K, F, act, nullptr);
+                       lda, row_of_slot, tile_expert, (const float*)w, mid, ldm, K, F, act, nullptr, limit);
   DA_CHECK_LAUNCH("moe_gated_ref");
   return 0;
 }
@@ -215,10 +214,10 @@ extern "C" int da_moe_down_ref(const void* mid, int ldm, int dtype, const int* r
   dim3 grid(da_ceil_div(width, MT), T_cap);
   if (dtype == DA_BF16)
     hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, MOE_DOWN>), grid, dim3(256), 0, (hipStream_t)stream,
-                       (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F, width, 0, nullptr);
+                       (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F, width, 0, nullptr, 0.f);
   else
     hipLaunchKernelGGL((moe_product_ref_kernel<float, MOE_DOWN>), grid, dim3(256), 0, (hipStream_t)stream,
-                       (const float*)mid, ldm, row_of_slot, tile_expert, (const float*)w, out, ldo, F, width, 0, nullptr);
+                       (const float*)mid, ldm, row_of_slot, tile_expert, (const float*)w, out, ldo, F, width, 0, nullptr, 0.f);
   DA_CHECK_LAUNCH("moe_down_ref");
   return 0;
 }
@@ -233,48 +232,56 @@ extern "C" int da_moe_up_ref(const void* a, int lda, int dtype, const int* row_o
   dim3 grid(da_ceil_div(F, MT), T_cap);
   if (dtype == DA_BF16)
     hipLaunchKernelGGL((moe_product_ref_kernel<bf16_t, MOE_UP>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)a,
-                       lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, slot_scale);
+                       lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, slot_scale, 0.f);
   else
     hipLaunchKernelGGL((moe_product_ref_kernel<float, MOE_UP>), grid, dim3(256), 0, (hipStream_t)stream, (const float*)a,
-                       lda, row_of_slot, tile_expert, (const float*)w, mid, ldm, K, F, act, slot_scale);
+                       lda, row_of_slot, tile_expert, (const float*)w, mid, ldm, K, F, act, slot_scale, 0.f);
   DA_CHECK_LAUNCH("moe_up_ref");
   return 0;
 }
 
-// The router of a mixture whose scores are logistic(z): every token's `top` largest (the lower index wins a tie),
-// ids[n, k] and weights[n, k] in descending order of the score.  `renorm`: the weights divided by their sum.
-__global__ void moe_top_logistic_kernel(const float* __restrict__ z, int ldz, int N, int E, int top, int renorm,
-                                        int* __restrict__ ids, float* __restrict__ weights) {
+// The router's choice from 32-bit logits z (+ bias, when given): every token's `top` largest (the lower index wins a
+// tie), ids[n, k] and weights[n, k] in descending order.  mode 0: the weights are logistic(z) (`renorm`: divided by
+// their sum); mode 1: the softmax over the chosen logits only.
+__global__ void moe_top_kernel(const float* __restrict__ z, int ldz, const void* __restrict__ bias, int bias_dtype, int N,
+                               int E, int top, int mode, int renorm, int* __restrict__ ids, float* __restrict__ weights) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= N) return;
   const float* row = z + (size_t)n * ldz;
-  float sum = 0.f;
+  float sum = 0.f, first = 0.f;
   for (int k = 0; k < top; ++k) {
     int best = -1;
     float bz = -INFINITY;
     for (int e = 0; e < E; ++e) {
-      const float v = row[e];
+      const float v = row[e] + (bias ? load_param(bias, bias_dtype, e) : 0.f);
       bool taken = false;
       for (int j = 0; j < k; ++j) taken |= ids[(size_t)n * top + j] == e;
       if (!taken && (best < 0 || v > bz)) { best = e; bz = v; }
     }
-    const float sc = 1.0f / (1.0f + expf(-bz));
+    if (k == 0) first = bz;
+    const float sc = mode == 1 ? expf(bz - first) : 1.0f / (1.0f + expf(-bz));
     ids[(size_t)n * top + k] = best;
     weights[(size_t)n * top + k] = sc;
     sum += sc;
   }
-  if (renorm)
+  if (renorm || mode == 1)
     for (int k = 0; k < top; ++k) weights[(size_t)n * top + k] /= sum;
+}
+
+extern "C" int da_moe_top(const float* z, int ldz, const void* bias, int bias_dtype, int N, int E, int top, int mode,
+                          int renorm, int* ids, float* weights, void* stream) {
+  DA_REQUIRE(N >= 0 && E > 0 && top > 0 && top <= E && ldz >= E, "moe_top: bad sizes");
+  DA_REQUIRE(mode == 0 || mode == 1, "moe_top: mode %d (0: logistic scores, 1: softmax over the chosen)", mode);
+  if (N == 0) return 0;
+  hipLaunchKernelGGL(moe_top_kernel, dim3(da_ceil_div(N, 64)), dim3(64), 0, (hipStream_t)stream, z, ldz, bias, bias_dtype, N,
+                     E, top, mode, renorm, ids, weights);
+  DA_CHECK_LAUNCH("moe_top");
+  return 0;
 }
 
 extern "C" int da_moe_top_logistic(const float* z, int ldz, int N, int E, int top, int renorm, int* ids, float* weights,
                                    void* stream) {
-  DA_REQUIRE(N >= 0 && E > 0 && top > 0 && top <= E && ldz >= E, "moe_top_logistic: bad sizes");
-  if (N == 0) return 0;
-  hipLaunchKernelGGL(moe_top_logistic_kernel, dim3(da_ceil_div(N, 64)), dim3(64), 0, (hipStream_t)stream, z, ldz, N, E, top,
-                     renorm, ids, weights);
-  DA_CHECK_LAUNCH("moe_top_logistic");
-  return 0;
+  return da_moe_top(z, ldz, nullptr, 0, N, E, top, 0, renorm, ids, weights, stream);
 }
 
 // slot_weight[slot_of_pair[i]] = weights[i]: a pair's weight where its slot's row is
@@ -336,7 +343,7 @@ template <int MODE>
 __global__ void __launch_bounds__(256)
 moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ row_of_slot,
                 const int* __restrict__ tile_expert, const bf16_t* __restrict__ w, void* __restrict__ out, int ldo,
-                int K, int F, int act, const float* __restrict__ slot_scale) {
+                int K, int F, int act, const float* __restrict__ slot_scale, float limit) {
   constexpr bool GATED = MODE == MOE_GATED, GATHER = MODE != MOE_DOWN;
   const int e = tile_expert[blockIdx.y];
   if (e < 0) return;
@@ -397,7 +404,7 @@ moe_mfma_kernel(const bf16_t* __restrict__ a, int lda, const int* __restrict__ r
       if (used < 0 || n0 + fr >= F) continue;
       const size_t o = (size_t)(m0 + i * 16 + row) * ldo + n0 + fr;
       const float sc = (GATHER && slot_scale) ? slot_scale[m0 + i * 16 + row] : 1.0f;
-      if (GATED) ((bf16_t*)out)[o] = f32_to_bf16(apply_act_bf16(sc * acc[i][0][r], act) * (sc * acc[i][GATED ? 1 : 0][r]));
+      if (GATED) ((bf16_t*)out)[o] = f32_to_bf16(gated_mid<true>(sc * acc[i][0][r], sc * acc[i][GATED ? 1 : 0][r], act, limit));
       else if (MODE == MOE_UP) ((bf16_t*)out)[o] = f32_to_bf16(apply_act_bf16(sc * acc[i][0][r], act));
       else ((float*)out)[o] = acc[i][0][r];
     }
@@ -412,13 +419,14 @@ static int moe_mfma_checks(const void* a, int lda, const void* w, int K, const c
 extern "C" int da_moe_tile_rows_mfma() { return MM_ROWS; }
 
 extern "C" int da_moe_gated_mfma(const void* a, int lda, const int* row_of_slot, const int* tile_expert, const void* w,
-                                 void* mid, int ldm, int T_cap, int K, int F, int act, void* stream) {
+                                 void* mid, int ldm, int T_cap, int K, int F, int act, float limit, void* stream) {
   DA_REQUIRE(T_cap >= 0 && K > 0 && F > 0 && lda >= K && ldm >= F, "moe_gated_mfma: bad sizes");
+  DA_REQUIRE(act != DA_ACT_GLU_CAPPED || limit > 0.f, "moe_gated_mfma: the capped form needs a positive limit");
   DA_REQUIRE(act >= DA_ACT_NONE && act <= DA_ACT_LAST, "moe_gated_mfma: unknown activation %d", act);
   if (moe_mfma_checks(a, lda, w, K, "moe_gated_mfma")) return 1;
   if (T_cap == 0) return 0;
   hipLaunchKernelGGL((moe_mfma_kernel<MOE_GATED>), dim3(da_ceil_div(F, MM_COLS), T_cap), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, nullptr);
+                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, nullptr, limit);
   DA_CHECK_LAUNCH("moe_gated_mfma");
   return 0;
 }
@@ -430,7 +438,7 @@ extern "C" int da_moe_up_mfma(const void* a, int lda, const int* row_of_slot, co
   if (moe_mfma_checks(a, lda, w, K, "moe_up_mfma")) return 1;
   if (T_cap == 0) return 0;
   hipLaunchKernelGGL((moe_mfma_kernel<MOE_UP>), dim3(da_ceil_div(F, MM_COLS), T_cap), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, slot_scale);
+                     (const bf16_t*)a, lda, row_of_slot, tile_expert, (const bf16_t*)w, mid, ldm, K, F, act, slot_scale, 0.f);
   DA_CHECK_LAUNCH("moe_up_mfma");
   return 0;
 }
@@ -442,7 +450,7 @@ extern "C" int da_moe_down_mfma(const void* mid, int ldm, const int* row_of_slot
   if (T_cap == 0) return 0;
   hipLaunchKernelGGL((moe_mfma_kernel<MOE_DOWN>), dim3(da_ceil_div(width, MM_COLS), T_cap), dim3(256), 0,
                      (hipStream_t)stream, (const bf16_t*)mid, ldm, row_of_slot, tile_expert, (const bf16_t*)w, out, ldo, F,
-                     width, 0, nullptr);
+                     width, 0, nullptr, 0.f);
   DA_CHECK_LAUNCH("moe_down_mfma");
   return 0;
 }

@@ -17,7 +17,9 @@ from ..profiler import KernelProfiler
 F32, BF16 = 0, 1
 MAX_HEAD_DIM = 256          # what the plain attention kernel takes; the matrix-core kernels: multiples of 16 up to it
 ACTIVATIONS = {None: 0, "none": 0, "gelu_new": 1, "gelu_pytorch_tanh": 1, "gelu": 2, "relu": 3, "silu": 4,
-               "relu2": 5}       # relu2: the square of max(x, 0)
+               "relu2": 5,       # relu2: the square of max(x, 0)
+               # only for a gated pair, with a limit c: g = min(gate, c), u = clamp(up, -c, c), g * logistic(1.702 g) * (u + 1)
+               "glu_capped": 6}
 
 
 class KernelError(RuntimeError):
@@ -97,8 +99,10 @@ _ARGTYPES = {
     "da_attn_prefill_rel": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _VP, _I, _I, _VP],
     "da_rmsnorm": [_VP, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
     "da_rmsnorm_add": [_VP, _VP, _I, _VP, _VP, _I, _F, _F, _VP, _I, _I, _I, _VP],
-    "da_attn_rel_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _F, _I, _VP, _I, _VP],
-    "da_attn_window": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _VP, _I, _I, _VP],
+    "da_attn_rel_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _F, _I, _F, _I, _VP, _VP, _I,
+                        _VP, _I, _VP],
+    "da_attn_window": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _VP, _VP, _I, _VP, _I, _I,
+                       _VP],
     "da_attn_window_takes": [_I, _I, _I],
     "da_attn_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _I, _VP, _VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _I, _VP],
     "da_delta_rule": [_VP, _I, _I, _I, _I, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I,
@@ -106,12 +110,15 @@ _ARGTYPES = {
     "da_delta_gate_norm": [_VP, _I, _VP, _I, _I, _VP, _I, _F, _I, _VP, _I, _I, _I, _I, _VP],
     "da_scale_add_rows": [_VP, _VP, _VP, _I, _I, _F, _VP],
     "da_kv_write_split": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
-    "da_gated_act": [_VP, _I, _I, _VP, _I, _I, _I, _I, _VP],
+    "da_gated_act": [_VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP],
+    "da_concat_rows": [_VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_retention": [_VP, _I, _I, _I, _I, _I, _VP, _F, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "da_moe_top": [_VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP],
     "da_softcap": [_VP, ctypes.c_long, _F, _VP],
     "da_moe_route": [_VP, _VP, _I, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP],
-    "da_moe_gated_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_moe_gated_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
     "da_moe_down_ref": [_VP, _I, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
-    "da_moe_gated_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
+    "da_moe_gated_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
     "da_moe_down_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _VP],
     "da_moe_gather": [_VP, _I, _VP, _VP, _I, _I, _VP, _VP],
     "da_gemm_bf16_grouped": [_VP, _I, _VP, _I, ctypes.c_long, _VP, _I, _VP, _I, _I, _I, _I, _I, _VP, _I],
@@ -119,10 +126,11 @@ _ARGTYPES = {
     "da_moe_up_mfma": [_VP, _I, _VP, _VP, _VP, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_moe_top_logistic": [_VP, _I, _I, _I, _I, _I, _VP, _VP, _VP],
     "da_moe_slot_weights": [_VP, _VP, _I, _VP, _VP],
-    "da_rotary": [_VP, _I, _I, _VP, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
-    "da_latent_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _VP, _VP, _VP, _I, _I, _VP, _I, _VP, _I, _I, _I, _VP],
-    "da_attn_latent_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _VP],
-    "da_attn_latent_mfma": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _I, _VP, ctypes.c_long, _VP],
+    "da_rotary": [_VP, _I, _I, _VP, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _VP],
+    "da_latent_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _VP, _VP, _VP, _I, _I, _F, _VP, _I, _VP, _I, _I, _I, _VP],
+    "da_attn_latent_ref": [_VP, _I, _VP, _I, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _F, _I, _VP, _VP, _I, _VP],
+    "da_attn_latent_mfma": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _F, _I, _VP, _I, _I, _VP, ctypes.c_long, _VP,
+                            _VP],
     "da_attn_latent_splits": [_I, _I, _I, _I],
     "da_attn_latent_mfma_takes": [_I, _I],
     "da_gemm_heads": [_VP, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _VP],
@@ -348,8 +356,9 @@ def scale_add_rows(src: torch.Tensor, scale: torch.Tensor, dst: torch.Tensor, mu
     return dst
 
 
-def gated_act(gu: torch.Tensor, mid: torch.Tensor, act: str) -> torch.Tensor:
-    """mid[r, j] = act(gu[r, j]) * gu[r, inner + j]: the halves of a fused gate | up product."""
+def gated_act(gu: torch.Tensor, mid: torch.Tensor, act: str, limit: float = 0.0) -> torch.Tensor:
+    """mid[r, j] = act(gu[r, j]) * gu[r, inner + j]: the halves of a fused gate | up product ("glu_capped" with its
+    ``limit``: see ``ACTIVATIONS``)."""
     _dev(gu, mid)
     _rows_2d(gu, "gu"); _rows_2d(mid, "mid")
     R, inner = mid.shape
@@ -358,8 +367,19 @@ def gated_act(gu: torch.Tensor, mid: torch.Tensor, act: str) -> torch.Tensor:
         raise KernelError(f"gated_act: unknown activation {act!r}")
     with _timed("gated_act", _nbytes(gu, mid), 10 * R * inner, "fp32"):
         _check(_lib().da_gated_act(_ptr(gu), gu.stride(0), _dt(gu), _ptr(mid), mid.stride(0), R, inner, ACTIVATIONS[act],
-                                   _stream()))
+                                   float(limit), _stream()))
     return mid
+
+
+def concat_rows(src: torch.Tensor, dst: torch.Tensor, col: int) -> torch.Tensor:
+    """dst[r, col : col + E] = src[r, :]: a 32-bit matrix [R, E] into columns of a wider matrix of either dtype."""
+    _dev(src, dst)
+    _rows_2d(dst, "dst")
+    _need(src.dtype == torch.float32 and src.dim() == 2 and src.is_contiguous(), "concat_rows: src must be contiguous float32")
+    R, E = src.shape
+    _need(dst.shape[0] >= R and 0 <= col and col + E <= dst.shape[1], "concat_rows: the columns leave the row")
+    _check(_lib().da_concat_rows(_ptr(src), _ptr(dst), _dt(dst), dst.stride(0), int(col), R, E, _stream()))
+    return dst
 
 
 def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
@@ -424,7 +444,7 @@ def _moe_common(a, row_of_slot, tile_expert, w, tiles, tile, name):
 
 
 def moe_gated_ref(a: torch.Tensor, row_of_slot: torch.Tensor, tile_expert: torch.Tensor, w: torch.Tensor,
-                  mid: torch.Tensor, tiles: int, act: str) -> torch.Tensor:
+                  mid: torch.Tensor, tiles: int, act: str, limit: float = 0.0) -> torch.Tensor:
     """mid[slot] = act(Wg_e a[row_of_slot[slot]]) * (Wu_e a[...]) for every used slot; w: [experts, 2 F, K]."""
     _moe_common(a, row_of_slot, tile_expert, w, tiles, MOE_TILE_ROWS, "moe_gated")
     K, F = a.shape[1], w.shape[1] // 2
@@ -435,7 +455,7 @@ def moe_gated_ref(a: torch.Tensor, row_of_slot: torch.Tensor, tile_expert: torch
         raise KernelError(f"moe_gated: unknown activation {act!r}")
     with _timed("moe_gated_plain", _nbytes(a, w, mid), 4 * tiles * MOE_TILE_ROWS * F * K, "fp32" if a.dtype == torch.float32 else "bf16"):
         _check(_lib().da_moe_gated_ref(_ptr(a), a.stride(0), _dt(a), _ptr(row_of_slot), _ptr(tile_expert), _ptr(w),
-                                       _ptr(mid), mid.stride(0), tiles, K, F, ACTIVATIONS[act], _stream()))
+                                       _ptr(mid), mid.stride(0), tiles, K, F, ACTIVATIONS[act], float(limit), _stream()))
     return mid
 
 
@@ -562,16 +582,20 @@ def kv_write_split(qkv: torch.Tensor, k_off: int, v_off: int, cache_slot: torch.
 def attention_rel_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
                       positions: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, v_head_dim: int, page: int,
                       scale: float, window: Optional[int], dist_bias: Optional[torch.Tensor], temp_coef: float,
-                      temp_every: int, out: torch.Tensor, softcap: float = 0.0, keep_first: int = 0) -> torch.Tensor:
+                      temp_every: int, out: torch.Tensor, softcap: float = 0.0, keep_first: int = 0,
+                      sink: Optional[torch.Tensor] = None, gate_col: int = -1) -> torch.Tensor:
     """Plain paged attention with a bias by distance (``dist_bias`` [Hq, n_dist] float32, the last column for every
     larger distance), a query temperature by position, values of their own size, a cap on the scores
-    (``softcap * tanh(score / softcap)``) and, with a window, ``keep_first`` first keys that stay visible."""
-    _dev(q, cache_slot, block_table, seq_of_token, positions, dist_bias, out)
+    (``softcap * tanh(score / softcap)``) and, with a window, ``keep_first`` first keys that stay visible.  ``sink``
+    (float32 [Hq]): exp(sink[h]) joins the softmax's denominator; ``gate_col`` >= 0: out * logistic(gate), the gate's
+    Hq * Dv entries lying in q's rows from that column on (q is then wider than its Hq * D query entries)."""
+    _dev(q, cache_slot, block_table, seq_of_token, positions, dist_bias, out, sink)
+    gate_ptr, gate_ld = _sink_gate_args(sink, gate_col, n_heads, n_heads * head_dim, n_heads * v_head_dim, q, "attention")
     _rows_2d(q, "q"); _rows_2d(out, "out")
     N = q.shape[0]
     _need(cache_slot.is_contiguous() and cache_page_elems(cache_slot) == n_kv_heads * page * (head_dim + v_head_dim),
           "attention: a page of the cache slot does not hold Hkv * page * (D + Dv) entries")
-    _need(q.shape[1] == n_heads * head_dim and out.shape[1] == n_heads * v_head_dim and out.shape[0] == N,
+    _need((q.shape[1] == n_heads * head_dim or gate_col >= 0) and out.shape[1] == n_heads * v_head_dim and out.shape[0] == N,
           "attention: q must be [N, Hq*D] and out [N, Hq*Dv]")
     _need(q.dtype == cache_slot.dtype == out.dtype, "attention: q, cache and out must share a dtype")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
@@ -586,9 +610,20 @@ def attention_rel_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: to
     _check(_lib().da_attn_rel_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table), block_table.shape[1],
                                   _ptr(seq_of_token), _ptr(positions), N, n_heads, n_kv_heads, head_dim, v_head_dim, page,
                                   float(scale), int(window or 0), _ptr(dist_bias), n_dist, float(temp_coef),
-                                  int(temp_every), float(softcap), int(keep_first if window else 0), _ptr(out),
-                                  out.stride(0), _stream()))
+                                  int(temp_every), float(softcap), int(keep_first if window else 0), _ptr(sink),
+                                  gate_ptr, gate_ld, _ptr(out), out.stride(0), _stream()))
     return out
+
+
+def _sink_gate_args(sink, gate_col, n_heads, q_cols, cols, q, name):
+    """Checks a sink vector and a gate that lies in q's rows; returns the gate's (address, row length)."""
+    if sink is not None:
+        _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == n_heads,
+              f"{name}: the sink must be float32 with one entry a query head")
+    if gate_col < 0:
+        return None, 0
+    _need(gate_col >= q_cols and gate_col + cols <= q.shape[1], f"{name}: the gate's columns leave q's rows or meet the queries")
+    return _ptr(q) + gate_col * q.element_size(), q.stride(0)
 
 
 # ------------------------------------------------------------------------------- sampling
@@ -1003,16 +1038,18 @@ def attention_prefill_rel(q: torch.Tensor, cache_slot: torch.Tensor, block_table
 def attention_window(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, q_start: torch.Tensor,
                      seq_lens: torch.Tensor, seq0: int, n_seqs: int, max_query_len: int, n_heads: int, n_kv_heads: int,
                      head_dim: int, v_head_dim: int, page: int, scale: float, window: Optional[int], keep_first: int,
-                     softcap: float, out: torch.Tensor, form: int = 0) -> torch.Tensor:
+                     softcap: float, out: torch.Tensor, form: int = 0, sink: Optional[torch.Tensor] = None,
+                     gate_col: int = -1) -> torch.Tensor:
     """Attention of the sequences ``seq0 .. seq0 + n_seqs - 1`` of a step on the matrix cores, in bfloat16, with keys and
     values of their own sizes, a cap on the scores and, with a window, ``keep_first`` first keys that stay visible.
     ``form``: 0 leaves the workgroup's row blocks to the kernel's rule; 1, 2 or 4 fixes them."""
-    _dev(q, cache_slot, block_table, q_start, seq_lens, out)
+    _dev(q, cache_slot, block_table, q_start, seq_lens, out, sink)
     _rows_2d(q, "q"); _rows_2d(out, "out")
+    gate_ptr, gate_ld = _sink_gate_args(sink, gate_col, n_heads, n_heads * head_dim, n_heads * v_head_dim, q, "attention_window")
     _need(q.dtype == cache_slot.dtype == out.dtype == torch.bfloat16, "attention_window: q, cache and out must be bfloat16")
     _need(cache_slot.is_contiguous() and cache_page_elems(cache_slot) == n_kv_heads * page * (head_dim + v_head_dim),
           "attention_window: a page of the cache slot does not hold Hkv * page * (D + Dv) entries")
-    _need(q.shape[1] == n_heads * head_dim and out.shape[1] == n_heads * v_head_dim and out.shape[0] == q.shape[0],
+    _need((q.shape[1] == n_heads * head_dim or gate_col >= 0) and out.shape[1] == n_heads * v_head_dim and out.shape[0] == q.shape[0],
           "attention_window: q must be [N, Hq*D] and out [N, Hq*Dv]")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous()
           and block_table.shape[0] >= seq0 + n_seqs, "attention_window: block_table must be contiguous int32 [S, max_blocks]")
@@ -1021,7 +1058,8 @@ def attention_window(q: torch.Tensor, cache_slot: torch.Tensor, block_table: tor
     _check(_lib().da_attn_window(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(block_table), block_table.shape[1],
                                  _ptr(q_start), _ptr(seq_lens), seq0, n_seqs, max_query_len, n_heads, n_kv_heads, head_dim,
                                  v_head_dim, page, float(scale), int(window or 0), int(keep_first if window else 0),
-                                 float(softcap), _ptr(out), out.stride(0), int(form), _stream()))
+                                 float(softcap), _ptr(sink), gate_ptr, gate_ld, _ptr(out),
+                                 out.stride(0), int(form), _stream()))
     return out
 
 
@@ -1032,9 +1070,12 @@ def attention_window_takes(head_dim: int, v_head_dim: int, page: int) -> bool:
 def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int, n_kv_heads: int,
                         head_dim: int, v_head_dim: int, scale: float, window: Optional[int],
                         dist_bias: Optional[torch.Tensor], temp_coef: float, temp_every: int,
-                        out: torch.Tensor, softcap: float = 0.0, keep_first: int = 0) -> torch.Tensor:
+                        out: torch.Tensor, softcap: float = 0.0, keep_first: int = 0,
+                        sink: Optional[torch.Tensor] = None, gate_col: int = -1) -> torch.Tensor:
     """Attention of every row of the step with a bias by distance, a query temperature, values of their own
-    size, a cap on the scores and first keys that a window keeps (each optional).  In bfloat16, with keys and values of one size that is a multiple of 16 up to 128 and a
+    size, a cap on the scores, first keys that a window keeps, a term without a key in the softmax's denominator
+    (``sink``) and a logistic gate on the result (``gate_col``: where the gate lies in q's rows), each optional; the last two go with the matrix-core
+    kernel for windows or the plain one.  In bfloat16, with keys and values of one size that is a multiple of 16 up to 128 and a
     bias row that fits the prefill kernel's LDS copy, the one-token sequences go to the decode kernel and the
     portions to the prefill kernel (their forms with these extras); a cap, kept first keys and values of another size
     go to the matrix-core kernel for those (head sizes up to 128, no bias table, no temperature); 32-bit, the reference
@@ -1063,7 +1104,7 @@ def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: i
                 2 * pairs * n_heads * (D + v_head_dim))
 
     tuned = (_MODE == "tuned" and q.dtype == torch.bfloat16 and v_head_dim == D and D % 16 == 0
-             and softcap == 0.0 and not (window and keep_first)
+             and softcap == 0.0 and not (window and keep_first) and sink is None and gate_col < 0
              and D <= PREFILL_REL_MAX_HEAD_DIM and cache_slot.dim() == 5 and q.stride(0) % 8 == 0
              and q.data_ptr() % 16 == 0 and (dist_bias is None or dist_bias.shape[1] <= PREFILL_REL_MAX_DIST))
     if tuned:
@@ -1086,23 +1127,44 @@ def paged_attention_rel(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: i
         if nd:
             with _timed("attention_window_decode", *cost(0, nd)):
                 attention_window(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, 0, nd, 1, n_heads, n_kv_heads, D,
-                                 v_head_dim, page, scale, window, keep_first, softcap, out)
+                                 v_head_dim, page, scale, window, keep_first, softcap, out, sink=sink, gate_col=gate_col)
         if ctx.n_seqs > nd:
             with _timed("attention_window", *cost(nd, ctx.n_seqs)):
                 attention_window(q, cache_slot, bt, ctx.q_start, ctx.seq_lens, nd, ctx.n_seqs - nd, ctx.max_query_len,
-                                 n_heads, n_kv_heads, D, v_head_dim, page, scale, window, keep_first, softcap, out)
+                                 n_heads, n_kv_heads, D, v_head_dim, page, scale, window, keep_first, softcap, out,
+                                 sink=sink, gate_col=gate_col)
         return out
     with _timed("attention_plain", *cost(0, ctx.n_seqs), "fp32" if q.dtype == torch.float32 else "bf16"):
         return attention_rel_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, n_kv_heads, head_dim,
-                                 v_head_dim, page, scale, window, dist_bias, temp_coef, temp_every, out, softcap, keep_first)
+                                 v_head_dim, page, scale, window, dist_bias, temp_coef, temp_every, out, softcap, keep_first,
+                                 sink=sink, gate_col=gate_col)
 
 
-def gated_linear(ctx, h: torch.Tensor, gate_up: torch.Tensor, mid: torch.Tensor, act: str) -> torch.Tensor:
+def gated_linear(ctx, h: torch.Tensor, gate_up: torch.Tensor, mid: torch.Tensor, act: str, limit: float = 0.0) -> torch.Tensor:
     """mid = act(h @ gate.T) * (h @ up.T) with gate | up as one matrix [2 inner, width]."""
     N, inner = mid.shape
     gu = ctx.buf("ff_gate_up", N, 2 * inner, h.dtype)
     linear(h, gate_up, None, gu)
-    return gated_act(gu, mid, act)
+    return gated_act(gu, mid, act, limit)
+
+
+def moe_top(z: torch.Tensor, bias: Optional[torch.Tensor], top: int, mode: str, renorm: bool, ids: torch.Tensor,
+            weights: torch.Tensor) -> None:
+    """Every row's ``top`` largest entries of z + bias (32-bit router logits; the lower index wins a tie): ids[n, k]
+    and weights[n, k] in descending order.  ``mode`` "logistic": weights logistic(z) (``renorm``: divided by their
+    sum); "softmax": the softmax over the chosen logits only."""
+    _dev(z, bias, ids, weights)
+    _rows_2d(z, "z")
+    N, E = z.shape
+    _need(z.dtype == torch.float32, "moe_top: router logits must be float32")
+    _need(1 <= top <= E, f"moe_top: top {top} of {E}")
+    _need(bias is None or (bias.is_contiguous() and bias.numel() == E), "moe_top: the bias has one entry an expert")
+    _need(mode in ("logistic", "softmax"), f"moe_top: unknown mode {mode!r}")
+    _need(ids.dtype == torch.int32 and ids.is_contiguous() and ids.numel() >= N * top and weights.dtype == torch.float32
+          and weights.is_contiguous() and weights.numel() >= N * top, "moe_top: ids int32 and weights float32, [N, top]")
+    with _timed("moe_top", N * E * 4 + N * top * 8, N * E * top, "fp32"):
+        _check(_lib().da_moe_top(_ptr(z), z.stride(0), _ptr(bias), _dt(bias) if bias is not None else 0, N, E, top,
+                                 1 if mode == "softmax" else 0, int(renorm), _ptr(ids), _ptr(weights), _stream()))
 
 
 def _moe_mfma_ok(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> bool:
@@ -1128,7 +1190,7 @@ def moe_top_logistic(z: torch.Tensor, top: int, renorm: bool, ids: torch.Tensor,
 def experts_forward(ctx, h: torch.Tensor, table: Optional[torch.Tensor], gate_up: torch.Tensor, down: torch.Tensor,
                     n_experts: int, top: int, weight: float, act: str, x: torch.Tensor, accumulate: bool,
                     ids: Optional[torch.Tensor] = None, pair_weights: Optional[torch.Tensor] = None,
-                    gated: bool = True, weight_input: bool = False) -> torch.Tensor:
+                    gated: bool = True, weight_input: bool = False, limit: float = 0.0) -> torch.Tensor:
     """x (+)= sum_k weight_k * expert_k(h) (or, with ``weight_input``, sum_k expert_k(weight_k * h)): route, two
     grouped products, combine.  The experts of a row come from ``table[token, k]`` or from ``ids[n, k]``; the
     weights are ``pair_weights[n, k]`` or the one ``weight``.  ``gated``: the first matrix of an expert is gate | up
@@ -1172,7 +1234,7 @@ def experts_forward(ctx, h: torch.Tensor, table: Optional[torch.Tensor], gate_up
                 _check(_lib().da_gemm_bf16_grouped(_ptr(hs), hs.stride(0), _ptr(gate_up), width, 2 * inner * width,
                                                    _ptr(tile_expert), tile, _ptr(gu), BF16, gu.stride(0), rows, 2 * inner, width,
                                                    _stream(), 0))
-            gated_act(gu, mid, act)
+            gated_act(gu, mid, act, limit)
         else:                      # the activation rides in the product's epilogue
             with _timed("experts_up", N * top * (width + inner) * 2 + _nbytes(gate_up), 2 * N * top * inner * width):
                 _check(_lib().da_gemm_bf16_grouped(_ptr(hs), hs.stride(0), _ptr(gate_up), width, inner * width,
@@ -1188,7 +1250,8 @@ def experts_forward(ctx, h: torch.Tensor, table: Optional[torch.Tensor], gate_up
         if gated:
             with _timed("experts_gated", nb, 4 * N * top * inner * width):
                 _check(_lib().da_moe_gated_mfma(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(gate_up),
-                                                _ptr(mid), mid.stride(0), tiles, width, inner, ACTIVATIONS[act], _stream()))
+                                                _ptr(mid), mid.stride(0), tiles, width, inner, ACTIVATIONS[act], float(limit),
+                                                _stream()))
         else:
             with _timed("experts_up", nb, 2 * N * top * inner * width):
                 _check(_lib().da_moe_up_mfma(_ptr(h), h.stride(0), _ptr(row_of_slot), _ptr(tile_expert), _ptr(gate_up),
@@ -1200,7 +1263,7 @@ def experts_forward(ctx, h: torch.Tensor, table: Optional[torch.Tensor], gate_up
                                            _ptr(pair_out), pair_out.stride(0), tiles, inner, width, _stream()))
     else:
         if gated:
-            moe_gated_ref(h, row_of_slot, tile_expert, gate_up, mid, tiles, act)
+            moe_gated_ref(h, row_of_slot, tile_expert, gate_up, mid, tiles, act, limit)
         else:
             _moe_common(h, row_of_slot, tile_expert, gate_up, tiles, MOE_TILE_ROWS, "moe_up")
             with _timed("moe_up_plain", _nbytes(h, gate_up, mid), 2 * tiles * MOE_TILE_ROWS * inner * width,
@@ -1244,7 +1307,8 @@ def linear_heads(a: torch.Tensor, a_head_stride: int, a_off: int, w: torch.Tenso
 
 
 def rotary(src: torch.Tensor, dst: torch.Tensor, positions: torch.Tensor, speeds: torch.Tensor, n_heads: int,
-           src_head_stride: int, dst_head_stride: int, width: int, dims: int, interleaved: bool = True) -> torch.Tensor:
+           src_head_stride: int, dst_head_stride: int, width: int, dims: int, interleaved: bool = True,
+           magnitude: float = 1.0) -> torch.Tensor:
     """dst[n, h, :width] = src[n, h, :width] with the first ``dims`` entries of every head turned in pairs by the angle
     positions[n] * speeds[i] (float64 [dims / 2]); pairs are (2i, 2i + 1) when ``interleaved``, else (i, i + dims/2).
     Heads start ``*_head_stride`` entries apart in a row; src and dst may be views into wider rows."""
@@ -1259,7 +1323,8 @@ def rotary(src: torch.Tensor, dst: torch.Tensor, positions: torch.Tensor, speeds
           "rotary: the heads leave the row")
     with _timed("rotary", 2 * N * n_heads * width * src.element_size(), 3 * N * n_heads * dims, "fp32"):
         _check(_lib().da_rotary(_ptr(src), src.stride(0), src_head_stride, _ptr(dst), dst.stride(0), dst_head_stride,
-                                _dt(src), _ptr(positions), _ptr(speeds), N, n_heads, width, dims, int(interleaved), _stream()))
+                                _dt(src), _ptr(positions), _ptr(speeds), N, n_heads, width, dims, int(interleaved),
+                                float(magnitude), _stream()))
     return dst
 
 
@@ -1276,7 +1341,7 @@ def latent_cache_row(cache_slot: torch.Tensor, page: int) -> int:
 def latent_prepare(down: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, q_gain: Optional[torch.Tensor],
                    kv_gain: torch.Tensor, eps: float, positions: torch.Tensor, slot_map: Optional[torch.Tensor],
                    speeds: torch.Tensor, dims: int, interleaved: bool, cq: Optional[torch.Tensor],
-                   cache_slot: torch.Tensor, page: int) -> None:
+                   cache_slot: torch.Tensor, page: int, magnitude: float = 1.0) -> None:
     """From rows [ query latent (q_rank) | latent (kv_rank) | key piece (rot_dim) ] of ``down``: cq = rms(query
     latent) * q_gain; the cache row slot_map[n] = [ rms(latent) * kv_gain | the key piece turned by the position ]."""
     _dev(down, q_gain, kv_gain, positions, slot_map, speeds, cq, cache_slot)
@@ -1296,17 +1361,18 @@ def latent_prepare(down: torch.Tensor, q_rank: int, kv_rank: int, rot_dim: int, 
     with _timed("latent_prepare", N * (q_rank + kv_rank + rot_dim) * (down.element_size() + cache_slot.element_size()), 6 * N * (q_rank + kv_rank + rot_dim), "fp32"):
         _check(_lib().da_latent_prepare(_ptr(down), _dt(down), down.stride(0), q_rank, kv_rank, rot_dim, _ptr(q_gain),
                                         _dt(q_gain) if q_gain is not None else 0, _ptr(kv_gain), _dt(kv_gain), float(eps),
-                                        _ptr(positions), _ptr(slot_map), _ptr(speeds), dims, int(interleaved), _ptr(cq),
+                                        _ptr(positions), _ptr(slot_map), _ptr(speeds), dims, int(interleaved), float(magnitude), _ptr(cq),
                                         cq.stride(0) if cq is not None else 0, _ptr(cache_slot), _dt(cache_slot), page, N,
                                         _stream()))
 
 
 def attention_latent_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table: torch.Tensor, seq_of_token: torch.Tensor,
                          positions: torch.Tensor, n_heads: int, row_dim: int, v_dim: int, page: int, scale: float,
-                         window: Optional[int], out: torch.Tensor) -> torch.Tensor:
+                         window: Optional[int], out: torch.Tensor, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Plain attention over a latent cache: q [N, Hq * row_dim] (the key maps folded in), out [N, Hq * v_dim] = the
-    weighted sums of the rows' first v_dim entries."""
-    _dev(q, cache_slot, block_table, seq_of_token, positions, out)
+    weighted sums of the rows' first v_dim entries.  ``sink`` (float32 [Hq]): exp(sink[h]) joins the denominator."""
+    _dev(q, cache_slot, block_table, seq_of_token, positions, out, sink)
+    _sink_gate_args(sink, -1, n_heads, 0, 0, q, "attention_latent")
     _rows_2d(q, "q"); _rows_2d(out, "out")
     N = q.shape[0]
     _need(cache_slot.is_contiguous() and latent_cache_row(cache_slot, page) == row_dim, "attention_latent: the cache rows differ from q's")
@@ -1319,13 +1385,14 @@ def attention_latent_ref(q: torch.Tensor, cache_slot: torch.Tensor, block_table:
           and positions.numel() >= N, "attention_latent: ids must be int32, one a row")
     _check(_lib().da_attn_latent_ref(_ptr(q), q.stride(0), _ptr(cache_slot), _dt(q), _ptr(block_table), block_table.shape[1],
                                      _ptr(seq_of_token), _ptr(positions), N, n_heads, row_dim, v_dim, page, float(scale),
-                                     int(window or 0), _ptr(out), out.stride(0), _stream()))
+                                     int(window or 0), _ptr(sink), _ptr(out), out.stride(0), _stream()))
     return out
 
 
 def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group: int, n_heads: int, row_dim: int,
-                           v_dim: int, scale: float, window: Optional[int], out: torch.Tensor) -> torch.Tensor:
-    """Attention of every row of the step over its sequence's latent rows."""
+                           v_dim: int, scale: float, window: Optional[int], out: torch.Tensor,
+                           sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of every row of the step over its sequence's latent rows (``sink``: see ``attention_latent_ref``)."""
     bt = ctx.block_tables[group]
     page = ctx.cache.page_size
     el = cache_slot.element_size()
@@ -1338,16 +1405,20 @@ def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group
         for s_ in range(first, ctx.n_seqs if last is None else last):
             t = starts[s_ + 1] - starts[s_]
             n = lens[s_]
-            keys += n
+            keys += min(n, window + t) if window else n
             rows += t
-            pairs += sum(n - t + i + 1 for i in range(t)) if t > 1 else n
+            if window:
+                pairs += sum(min(n - t + i + 1, window) for i in range(t))
+            else:
+                pairs += sum(n - t + i + 1 for i in range(t)) if t > 1 else n
         return keys * row_dim * el + rows * n_heads * (row_dim + v_dim) * el, 2 * pairs * n_heads * (row_dim + v_dim)
 
     if (_MODE == "tuned" and q.dtype == torch.bfloat16 and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0
             and bool(_lib().da_attn_latent_mfma_takes(row_dim, v_dim))):
         # prompt portions and decoded tokens alike: the query rows of a workgroup are (token, head) pairs
-        _dev(q, cache_slot, bt, out)
+        _dev(q, cache_slot, bt, out, sink)
         _rows_2d(q, "q"); _rows_2d(out, "out")
+        _sink_gate_args(sink, -1, n_heads, 0, 0, q, "attention_latent")
         _need(cache_slot.is_contiguous() and cache_slot.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
               and latent_cache_row(cache_slot, page) == row_dim, "attention_latent: a bfloat16 cache of rows like q's")
         _need(q.shape[1] == n_heads * row_dim and out.shape[1] == n_heads * v_dim and out.shape[0] == q.shape[0],
@@ -1360,7 +1431,7 @@ def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group
             _check(_lib().da_attn_latent_mfma(_ptr(q), q.stride(0), _ptr(cache_slot), _ptr(bt), bt.shape[1], _ptr(ctx.q_start),
                                               _ptr(ctx.seq_lens), seq0, n_seqs, max_q, n_heads, row_dim, v_dim, page,
                                               float(scale), int(window or 0), _ptr(out), out.stride(0), n_splits, _ptr(ws),
-                                              0 if ws is None else ws.numel(), _stream()))
+                                              0 if ws is None else ws.numel(), _ptr(sink), _stream()))
         if nd:                 # one-token sequences: the keys of a token's heads shared out over workgroups
             n_splits = int(_lib().da_attn_latent_splits(nd, n_heads, bt.shape[1], page))
             ws = None
@@ -1374,7 +1445,38 @@ def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group
         return out
     with _timed("attention_latent_plain", *cost(), "fp32" if q.dtype == torch.float32 else "bf16"):
         return attention_latent_ref(q, cache_slot, bt, ctx.seq_of_token, ctx.positions, n_heads, row_dim, v_dim, page,
-                                    scale, window, out)
+                                    scale, window, out, sink=sink)
+
+
+# ------------------------------------------------------------------------------- retention
+RETENTION_MAX_DIM = 256      # key entries a head of the retention kernel (csrc/retention.hip)
+
+
+def retention(ctx, qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torch.Tensor, k_scale: float,
+              state: torch.Tensor, o: torch.Tensor, n_heads: int, head_dim: int, v_head_dim: int,
+              write: bool = True) -> torch.Tensor:
+    """Per head S <- decay[h] S + k v^T, o = S^T q over every sequence of the step, token by token (csrc/retention.hip).
+    ``qkv`` [N, ...] holds the turned q and k (H * D entries each, from columns ``q_off`` and ``k_off``) and v (H * Dv
+    from ``v_off``) in the step's dtype; k is multiplied by ``k_scale``; ``decay`` float32 [H]; ``state`` [slots, >= H * Dv
+    * D] 32-bit is read at each portion's start and, with ``write``, written at its end; ``o`` [N, H * Dv] 32-bit."""
+    _dev(qkv, decay, state, o)
+    _rows_2d(qkv, "qkv"); _rows_2d(o, "o")
+    N = qkv.shape[0]
+    H, D, Dv = n_heads, head_dim, v_head_dim
+    ld = _state_args(state, "retention")
+    _need(1 <= D <= RETENTION_MAX_DIM, f"retention: a key size of {D} is outside 1..{RETENTION_MAX_DIM}")
+    _need(min(q_off, k_off, v_off) >= 0 and max(q_off, k_off) + H * D <= qkv.shape[1] and v_off + H * Dv <= qkv.shape[1],
+          "retention: q, k and v leave the row")
+    _need(o.dtype == torch.float32 and o.shape[0] == N and o.shape[1] >= H * Dv, "retention: o must be float32 [N, H * Dv]")
+    _need(decay.dtype == torch.float32 and decay.is_contiguous() and decay.numel() == H, "retention: decay must be float32 [H]")
+    _need(ld >= H * Dv * D, "retention: the state row is too short")
+    _need(ctx.q_start.numel() >= ctx.n_seqs + 1 and ctx.state_slots.numel() >= ctx.n_seqs, "retention: the step's arrays are too short")
+    nb = N * ((2 * H * D + H * Dv) * qkv.element_size() + H * Dv * 4) + 2 * ctx.n_seqs * H * Dv * D * 4
+    with _timed("retention", nb, 4 * N * H * D * Dv, "fp32"):
+        _check(_lib().da_retention(_ptr(qkv), _dt(qkv), qkv.stride(0), int(q_off), int(k_off), int(v_off), _ptr(decay),
+                                   float(k_scale), _ptr(state), ld, _ptr(ctx.state_slots), _ptr(ctx.q_start), _ptr(o),
+                                   o.stride(0), ctx.n_seqs, H, D, Dv, int(bool(write)), _stream()))
+    return o
 
 
 # ------------------------------------------------------------------------------- short filter and scan

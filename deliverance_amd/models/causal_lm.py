@@ -38,6 +38,14 @@ class CausalLM:
             build_norm(config.final_norm, params["final_norm"], dtype, device)
         embed_norm = getattr(config, "embed_norm", None)
         self.embed_norm = None if embed_norm is None else build_norm(embed_norm, params["embed_norm"], dtype, device)
+        # W [width, 2 width] for run-order entries that mix the stream with the embedding output
+        self.input_mix = None
+        if getattr(config, "input_mix", False):
+            self.input_mix = to_matrix(params["input_mix"]["weight"], dtype, device)
+            if tuple(self.input_mix.shape) != (config.width, 2 * config.width):
+                raise ValueError(f"the input mix is {list(self.input_mix.shape)}, expected {[config.width, 2 * config.width]}")
+        elif any(getattr(c, "mix_input", False) for c in config.schedule):
+            raise ValueError("the run order mixes the stream with the embedding output, but the model has no matrix for it")
         head = params["head"]["weight"]
         if head is emb["tokens"] and self.token_table.dtype == dtype:
             self.head_weight = self.token_table            # tied: one buffer, two uses
@@ -94,7 +102,15 @@ class CausalLM:
         debug = ctx.debug_hook is not None          # the reference's stages: AbstractModel.java:1100,1107
         if debug:
             ctx.emit(-1, "input", x)
+        both = None
+        if self.input_mix is not None:
+            # [stream | embedding output] in the compute dtype; the right half is written once a step
+            both = ctx.buf("input_mix", N, 2 * self.config.width, ctx.dtype)
+            ops.concat_rows(x, both, self.config.width)
         for call in self.config.schedule:
+            if getattr(call, "mix_input", False):       # x <- W [x; embedding output]
+                ops.concat_rows(x, both, 0)
+                ops.linear(both, self.input_mix, None, x)
             self.blocks[call.layer].forward(ctx, x, call)
             if debug:
                 ctx.emit(call.layer, "layer_output", x)

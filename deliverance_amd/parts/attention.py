@@ -10,7 +10,11 @@ buckets that the mixer writes out once as a table by distance), a query temperat
 the position (``query_temperature``), a root-mean-square norm of queries and keys before the rotation
 (``qk_norm``: over a token's whole projection or head by head), a cap on the scores (``score_softcap``:
 cap * tanh(score / cap)), and first keys of a sequence that a window never leaves behind (``keep_first``:
-position i sees j <= i when i - j < window or j < keep_first).
+position i sees j <= i when i - j < window or j < keep_first), values that are the keys before their rotation
+(``values_are_keys``: the caller stacks the key matrix twice into the one projection, so the product gives them), a
+term without key or value in the softmax's denominator (``sink``: exp(0), or exp of a learned number per head), and a
+logistic gate of one more projection of the input on the heads' results (``out_gate``: its rows are stacked behind
+q | k | v in the same product).
 Reference: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:226-420
 (projections :266-291, cache write :315-336, scores/softmax/weighted sum :458-532, output
 projection :385-408); the residual add is TransformerBlock.java:176.
@@ -65,14 +69,31 @@ class CausalSelfAttention(Mixer):
         self.v_cols = self.n_kv_heads * self.v_head_dim
         self.o_cols = self.n_heads * self.v_head_dim
         self.qkv_cols = self.q_cols + self.kv_cols + self.v_cols
+        self.out_gate = getattr(spec, "out_gate", None)
+        if self.out_gate not in (None, "sigmoid"):
+            raise ValueError(f"an output gate is 'sigmoid' or None, not {self.out_gate!r}")
+        if getattr(spec, "values_are_keys", False) and self.v_head_dim != self.head_dim:
+            raise ValueError(f"values that are the keys have the keys' size {self.head_dim}, not {self.v_head_dim}")
+        self.gate_off = self.qkv_cols                 # the gate's columns in the projection's rows, when there is one
+        self.proj_cols = self.qkv_cols + (self.o_cols if self.out_gate else 0)
         self.scale = float(spec.scale)
         self.window = spec.window
         self.qkv_weight = to_matrix(params["qkv_weight"], dtype, device)
         self.out_weight = to_matrix(params["out_weight"], dtype, device)
         self.qkv_bias = to_vector(params.get("qkv_bias"), dtype, device) if spec.qkv_bias else None
         self.out_bias = to_vector(params.get("out_bias"), dtype, device) if spec.out_bias else None
-        if tuple(self.qkv_weight.shape) != (self.qkv_cols, spec.width):
-            raise ValueError(f"qkv weight is {list(self.qkv_weight.shape)}, expected {[self.qkv_cols, spec.width]}")
+        if tuple(self.qkv_weight.shape) != (self.proj_cols, spec.width):
+            raise ValueError(f"qkv weight is {list(self.qkv_weight.shape)}, expected {[self.proj_cols, spec.width]}")
+        sink = getattr(spec, "sink", None)
+        if sink not in (None, "zero", "learned"):
+            raise ValueError(f"a sink is 'zero', 'learned' or None, not {sink!r}")
+        self.sink = None                              # 32-bit, one a query head
+        if sink == "zero":
+            self.sink = torch.zeros(self.n_heads, dtype=torch.float32, device=device)
+        elif sink == "learned":
+            self.sink = params["sink"].to(device=device, dtype=torch.float32).contiguous()
+            if self.sink.numel() != self.n_heads:
+                raise ValueError(f"the sink has {self.sink.numel()} entries for {self.n_heads} heads")
         if tuple(self.out_weight.shape) != (spec.width, self.o_cols):
             raise ValueError(f"output weight is {list(self.out_weight.shape)}, expected {[spec.width, self.o_cols]}")
         # the extras: a table by distance [heads, max_distance + 1] (32-bit) and the temperature's constants
@@ -103,7 +124,7 @@ class CausalSelfAttention(Mixer):
                 raise ValueError(f"query and key gains have {self.q_gain.numel()} and {self.k_gain.numel()} entries, "
                                  f"expected {nq} and {nk}")
         self.extras = (self.dist_bias is not None or self.temp_every > 0 or self.v_head_dim != self.head_dim
-                       or self.softcap > 0.0 or self.keep_first > 0)
+                       or self.softcap > 0.0 or self.keep_first > 0 or self.sink is not None or self.out_gate is not None)
         self.position = None
         if spec.position is not None and spec.position.kind != "none":
             self.position = build_position(spec.position, params.get("position", {}), dtype, device)
@@ -115,7 +136,8 @@ class CausalSelfAttention(Mixer):
     def _epilogue_write(self) -> bool:
         """Whether the q|k|v product may write keys and values to the cache itself (its epilogue assumes
         keys and values of one size)."""
-        return self.position is None and self.v_head_dim == self.head_dim and self.qk_norm is None
+        return (self.position is None and self.v_head_dim == self.head_dim and self.qk_norm is None
+                and self.out_gate is None)
 
     normed_into = True
 
@@ -143,7 +165,7 @@ class CausalSelfAttention(Mixer):
 
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
         N = h.shape[0]
-        qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
+        qkv = ctx.buf("qkv", N, self.proj_cols, ctx.dtype)
         slot = ctx.cache.kv[call.cache]
         group = ctx.group_of(call.cache)
         if self._epilogue_write() and call.write:
@@ -153,6 +175,8 @@ class CausalSelfAttention(Mixer):
         elif self.qk_norm is not None:
             # the norms act on the product's unrounded 32-bit sums; one kernel then normalises queries and keys,
             # turns them by the position, stores the queries and writes keys and values to the cache
+            if self.out_gate is not None:
+                raise ValueError("an output gate beside a norm of queries and keys is not built")
             raw = ctx.buf("qkv_raw", N, self.qkv_cols, torch.float32)
             ops.linear(h, self.qkv_weight, self.qkv_bias, raw)
             rot = self.position if hasattr(self.position, "speeds") else None
@@ -181,15 +205,17 @@ class CausalSelfAttention(Mixer):
         N = qkv.shape[0]
         o = ctx.buf("attn_out", N, self.o_cols, ctx.dtype)
         if self.extras:
-            ops.paged_attention_rel(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.n_kv_heads, self.head_dim,
+            # with a gate, q is the projection's whole rows: queries first, the gate from ``gate_off`` on
+            ops.paged_attention_rel(ctx, qkv if self.out_gate else qkv[:, :self.q_cols], slot, group, self.n_heads, self.n_kv_heads, self.head_dim,
                                     self.v_head_dim, self.scale, self.window, self.dist_bias, self.temp_coef,
-                                    self.temp_every, o, softcap=self.softcap, keep_first=self.keep_first)
+                                    self.temp_every, o, softcap=self.softcap, keep_first=self.keep_first, sink=self.sink,
+                                    gate_col=self.gate_off if self.out_gate else -1)
         else:
             ops.paged_attention(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.scale, self.window, o)
         if ctx.debug_hook is not None:      # the reference's stage names (CausalSelfAttention.java:299-301,384)
             ctx.emit(call.layer, "query_projection", qkv[:, :self.q_cols])
             ctx.emit(call.layer, "key_projection", qkv[:, self.q_cols:self.q_cols + self.kv_cols])
-            ctx.emit(call.layer, "value_projection", qkv[:, self.q_cols + self.kv_cols:])
+            ctx.emit(call.layer, "value_projection", qkv[:, self.q_cols + self.kv_cols:self.qkv_cols])
             ctx.emit(call.layer, "attention_value", o)
             # the output projection before its bias (CausalSelfAttention.java:406), worked out once more for the hook
             ctx.emit(call.layer, "attention_output",

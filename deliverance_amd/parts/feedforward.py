@@ -56,8 +56,11 @@ class GatedFeedForward(FeedForward):
 
     def __init__(self, spec, params, dtype, device):
         self.width, self.inner, self.activation = spec.width, spec.inner, spec.activation
+        self.limit = float(getattr(spec, "limit", 0.0) or 0.0)
         if self.activation not in ops.ACTIVATIONS:
             raise ValueError(f"unknown activation {self.activation!r}")
+        if self.activation == "glu_capped" and not (self.limit > 0.0):
+            raise ValueError(f"the capped gated form needs a positive limit, found {self.limit}")
         self.gate_up_weight = to_matrix(params["gate_up_weight"], dtype, device)
         self.down_weight = to_matrix(params["down_weight"], dtype, device)
         if tuple(self.gate_up_weight.shape) != (2 * self.inner, self.width):
@@ -68,7 +71,7 @@ class GatedFeedForward(FeedForward):
     def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor) -> None:
         N = h.shape[0]
         mid = ctx.buf("ff_mid", N, self.inner, ctx.dtype)
-        ops.gated_linear(ctx, h, self.gate_up_weight, mid, self.activation)
+        ops.gated_linear(ctx, h, self.gate_up_weight, mid, self.activation, self.limit)
         ops.linear(mid, self.down_weight, None, x, accumulate=ctx.part_accumulate)
 
 
@@ -76,6 +79,8 @@ class ExpertsFeedForward(FeedForward):
     """A mixture of experts (``ExpertsFeedForwardSpec``).  The router says which ``top`` experts a token uses and
     with what weights.  ``token_table``: row ``token id`` of an integer table names them, each with weight 1 / top.
     ``logistic_top``: 32-bit logits from a matrix; the ``top`` largest logistic scores, which are the weights.
+    ``softmax_top``: 32-bit logits from a matrix and a bias; the ``top`` largest logits, weighted by the softmax over
+    just those.
     The step's (token, choice) pairs are laid out expert by expert on the device (``ops.moe_route``), two grouped
     products run over that layout, and the pairs' results are added up per token; a weight on the input scales
     the pair's row in the first product.  A shared expert, if any, runs as a dense feed-forward for every token.
@@ -91,8 +96,11 @@ class ExpertsFeedForward(FeedForward):
         self.renormalize = bool(getattr(spec, "renormalize", False))
         if self.activation not in ops.ACTIVATIONS:
             raise ValueError(f"unknown activation {self.activation!r}")
-        if self.router not in ("token_table", "logistic_top"):
-            raise ValueError(f"unknown router {self.router!r}; known: 'token_table', 'logistic_top'")
+        self.limit = float(getattr(spec, "limit", 0.0) or 0.0)
+        if self.router not in ("token_table", "logistic_top", "softmax_top"):
+            raise ValueError(f"unknown router {self.router!r}; known: 'token_table', 'logistic_top', 'softmax_top'")
+        if self.activation == "glu_capped" and not (self.gated and self.limit > 0.0):
+            raise ValueError(f"the capped gated form needs gated experts and a positive limit, found {self.limit}")
         if self.weight_on not in ("output", "input"):
             raise ValueError(f"a pair's weight goes on the 'output' or the 'input', not {self.weight_on!r}")
         if not (1 <= self.top <= self.n_experts):
@@ -121,10 +129,21 @@ class ExpertsFeedForward(FeedForward):
             self.router_weight = to_matrix(params["router_weight"], dtype, device)     # [experts, width]
             if tuple(self.router_weight.shape) != (self.n_experts, self.width):
                 raise ValueError(f"router weight is {list(self.router_weight.shape)}, expected {[self.n_experts, self.width]}")
+        self.router_bias = None
+        if getattr(spec, "router_bias", False):
+            self.router_bias = params["router_bias"].to(device=device, dtype=torch.float32).contiguous()
+            if self.router_bias.numel() != self.n_experts:
+                raise ValueError(f"the router's bias has {self.router_bias.numel()} entries for {self.n_experts} experts")
         self.weight = 1.0 / self.top
         self.last_choice = None
         self.shared = None
-        if getattr(spec, "shared_inner", 0):
+        if getattr(spec, "shared_inner", 0) and getattr(spec, "shared_gated", False):
+            from ..config.specs import GatedFeedForwardSpec
+            self.shared = GatedFeedForward(
+                GatedFeedForwardSpec("gated", self.width, spec.shared_inner, spec.shared_activation or self.activation,
+                                     limit=float(getattr(spec, "shared_limit", 0.0) or 0.0)),
+                {"gate_up_weight": params["shared_gate_up_weight"], "down_weight": params["shared_down_weight"]}, dtype, device)
+        elif getattr(spec, "shared_inner", 0):
             from ..config.specs import DenseFeedForwardSpec
             self.shared = DenseFeedForward(
                 DenseFeedForwardSpec("dense", self.width, spec.shared_inner, spec.shared_activation or self.activation,
@@ -139,11 +158,15 @@ class ExpertsFeedForward(FeedForward):
             ops.linear(h, self.router_weight, None, z)
             ids = ctx.buf("moe_ids", N, self.top, torch.int32)
             weights = ctx.buf("moe_weights", N, self.top, torch.float32)
-            ops.moe_top_logistic(z, self.top, self.renormalize, ids, weights)
+            if self.router == "softmax_top":
+                ops.moe_top(z, self.router_bias, self.top, "softmax", False, ids, weights)
+            else:
+                ops.moe_top(z, self.router_bias, self.top, "logistic", self.renormalize, ids, weights)
         self.last_choice = ids if ctx.debug_hook is not None else None      # handed to the layer debug hook
         ops.experts_forward(ctx, h, self.table, self.gate_up_weight, self.down_weight, self.n_experts, self.top,
                             self.weight, self.activation, x, accumulate=ctx.part_accumulate, ids=ids,
-                            pair_weights=weights, gated=self.gated, weight_input=self.weight_on == "input")
+                            pair_weights=weights, gated=self.gated, weight_input=self.weight_on == "input",
+                            limit=self.limit)
         if self.shared is not None:
             keep = ctx.part_accumulate
             ctx.part_accumulate = True          # the shared expert joins the experts' sum, stored or added above

@@ -1,5 +1,8 @@
 """Attention over one narrow vector a token, as a mixer (``LatentAttentionSpec``).
 
+Optional: a window (``spec.window``: position i sees j when 0 <= i - j < window), and a learned number per head whose
+exponential joins the softmax's denominator without a key or a value (``spec.sink``).
+
 What a token leaves in the cache is the normalised latent c (``kv_rank`` entries) and one key piece turned by
 its position (``rot_dim`` entries); every head's keys and values are linear maps of c.  The maps are never
 applied to cached rows: a head's key map is folded into its query (q'_h = [Wk_h^T q_h | turned q_h], so that
@@ -51,6 +54,10 @@ class LatentAttention(Mixer):
         self.v_up = to_matrix(shaped("v_up_weight", (H * self.dv, self.kv_rank)).reshape(H, self.dv, self.kv_rank),
                               dtype, device)                                                     # [H, dv, kv_rank]
         self.out_weight = to_matrix(shaped("out_weight", (E, H * self.dv)), dtype, device)
+        # exp(sink_h) in the softmax's denominator: 32-bit, one a head
+        self.sink = None
+        if getattr(spec, "sink", False):
+            self.sink = shaped("sink", (H,)).to(device=device, dtype=torch.float32).contiguous()
         self.rotary = build_position(spec.rotary, {}, dtype, device)
         if self.rotary.dims > self.dr:
             raise ValueError(f"{self.rotary.dims} turned entries, the rotated piece has {self.dr}")
@@ -85,7 +92,7 @@ class LatentAttention(Mixer):
         cq = ctx.buf("latent_cq", N, self.q_rank, ctx.dtype)
         ops.latent_prepare(down, self.q_rank, self.kv_rank, self.dr, self.q_gain, self.kv_gain, self.eps, ctx.positions,
                            ctx.slot_maps[group] if call.write else None, self.rotary.speeds, self.rotary.dims,
-                           self.rotary.interleaved, cq, slot, ctx.cache.page_size)
+                           self.rotary.interleaved, cq, slot, ctx.cache.page_size, magnitude=self.rotary.magnitude)
         q = ctx.buf("latent_q", N, H * qd, ctx.dtype)
         ops.linear(cq, self.q_up_weight, None, q)
         # q'_h = [Wk_h^T q_h[:dn] | turned q_h[dn:]]
@@ -93,7 +100,8 @@ class LatentAttention(Mixer):
         ops.linear_heads(q, qd, 0, self.k_fold, qf, self.row_dim, 0)
         self.rotary.apply(ctx, q[:, self.dn:], qf[:, self.kv_rank:], H, qd, self.row_dim, self.dr)
         mix = ctx.buf("latent_mix", N, H * self.kv_rank, ctx.dtype)
-        ops.paged_attention_latent(ctx, qf, slot, group, H, self.row_dim, self.kv_rank, self.scale, self.window, mix)
+        ops.paged_attention_latent(ctx, qf, slot, group, H, self.row_dim, self.kv_rank, self.scale, self.window, mix,
+                                   sink=self.sink)
         o = ctx.buf("attn_out", N, H * self.dv, ctx.dtype)
         ops.linear_heads(mix, self.kv_rank, 0, self.v_up, o, self.dv, 0)
         if ctx.debug_hook is not None:
