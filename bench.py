@@ -18,7 +18,7 @@ its fraction of the roofline; `--no-extra` leaves those two out.  Prints ONE JSO
 vocabulary, feed-forward parameters that a token uses): decode at batch 1, 8 and 64 and the prefill of 2 x 1,024
 tokens for both, at the layer sizes of GPT-2 124M and 355M, one JSON line; with `--profile-stages` also both
 models' kernel tables (stderr).  `--design pedatar` does the same for a third design beside Virudra (the closest
-of the engine's models to it), and `--design pafolorn` for a fourth beside Pedatar.
+of the engine's models to it), `--design pafolorn` for a fourth beside Pedatar, and `--design salivik` for a fifth beside Pedatar.
 """
 import argparse
 import json
@@ -340,12 +340,137 @@ def pafolorn_compare(args):
     return 0
 
 
+def salivik_config(name, n_positions=1024):
+    """A Salivik of GPT-2 ``name``'s sizes: as many layer runs, with latent attention, attention whose keys are its values
+    and retention in turn.  Latent attention as in ``pedatar_config`` (GPT-2's heads, 48 + 16 query entries, values of 64,
+    a query latent of half the width, a latent of a quarter of the width beside a key piece of 16) with a window of 512
+    keys, a learned sink and ramped speeds.  Attention: GPT-2's heads of 64 entries on a quarter as many key heads, the
+    first 32 entries rotated, a window of 512.  Retention: GPT-2's heads with 64 key and 64 value entries.  Feed-forward:
+    8 capped gated experts of 2/3 of the width (2 a token) and a shared one of 4/3 of the width, which hold what
+    Pedatar's ungated ones hold for a token.  The first three layers run twice (a loop), so the stored layers are three
+    fewer than the runs."""
+    g = MODELS[name]
+    E, H = g["n_embd"], g["n_head"]
+    lat = {"heads": H, "dim": 48, "rot_dim": 16, "vdim": 64, "q_rank": E // 2, "kv_rank": E // 4, "scale": 64 ** -0.5,
+           "mask": {"size": 512}, "rot": {"base": 10000.0, "dims": 16, "scaling": {"factor": 4.0, "original": 256, "fast": 32.0, "slow": 1.0}}}
+    att = {"heads": H, "kv_heads": H // 4, "dim": 64, "vdim": 64, "scale": 64 ** -0.5, "mask": {"size": 512},
+           "rot": {"base": 10000.0, "dims": 32}}
+    ret = {"heads": H, "dim": 64, "vdim": 64, "decay": [1.0 - 2.0 ** (-5 - i % 8) for i in range(H)], "rot": {"base": 10000.0, "dims": 64}}
+    f, fs = (2 * E // 3) // 8 * 8, (4 * E // 3) // 8 * 8
+    mlp = {"kind": "moe", "expert": {"ff": f, "limit": 7.0}, "router": {"experts": 8, "top": 2}, "shared": {"ff": fs, "limit": 7.0}}
+    kinds = (("latent_attention", lat), ("attention", att), ("retention", ret))
+    layers = [{"type": kinds[i % 3][0], "mixer": kinds[i % 3][1], "mlp": mlp} for i in range(g["n_layer"] - 3)]
+    return {"architecture": "Salivik", "vocab": 50257, "width": E, "norm": {"eps": 1e-5}, "layers": layers,
+            "loop": {"start": 0, "stop": 3, "times": 2}, "max_positions": n_positions,
+            # what decode_run and prefill_run read
+            "vocab_size": 50257, "n_positions": n_positions, "n_layer": g["n_layer"], "n_embd": E}
+
+
+def _salivik_runs(c):
+    lp = c["loop"]
+    order = list(range(lp["start"])) + list(range(lp["start"], lp["stop"])) * lp["times"] + list(range(lp["stop"], len(c["layers"])))
+    return [c["layers"][i] for i in order]
+
+
+def _salivik_layer_params(c, L, experts_used):
+    E, m = c["width"], L["mixer"]
+    if L["type"] == "latent_attention":
+        H, qd = m["heads"], m["dim"] + m["rot_dim"]
+        n = E * (m["q_rank"] + m["kv_rank"] + m["rot_dim"]) + m["q_rank"] * H * qd + m["kv_rank"] * H * (m["dim"] + m["vdim"]) + H * m["vdim"] * E
+    elif L["type"] == "attention":
+        n = E * m["dim"] * (3 * m["heads"] + m["kv_heads"])
+    else:
+        n = E * m["heads"] * (2 * m["dim"] + 3 * m["vdim"])
+    f = L["mlp"]
+    return n + 3 * E * (experts_used * f["expert"]["ff"] + f["shared"]["ff"]) + f["router"]["experts"] * E
+
+
+def salivik_step_bytes(c, el, batch, ctx_mean):
+    """What a decode step must read: every matrix of every run once (of the experts as many as ``batch`` tokens can
+    choose; a looped layer's matrices are read again in its second pass), the keys that the windows see, and the
+    retention states (read and written, 32-bit)."""
+    n, extra = c["vocab"] * c["width"] + 2 * c["width"] ** 2 * c["loop"]["times"], 0
+    for L in _salivik_runs(c):
+        f = L["mlp"]["router"]
+        n += _salivik_layer_params(c, L, min(f["experts"], f["top"] * batch))
+        m = L["mixer"]
+        if L["type"] == "latent_attention":
+            extra += batch * min(ctx_mean, m["mask"]["size"]) * (m["kv_rank"] + m["rot_dim"]) * el
+        elif L["type"] == "attention":
+            extra += batch * min(ctx_mean, m["mask"]["size"]) * m["kv_heads"] * 2 * m["dim"] * el
+        else:
+            extra += batch * 2 * 4 * m["heads"] * m["dim"] * m["vdim"]
+    return n * el + extra
+
+
+def salivik_step_flops(c, seq_lens_new):
+    """Matrix-product flops of a step (the parameters a token uses, twice), the attentions' two products over the keys
+    that each row sees, and the retention's four operations a state entry and token."""
+    n = sum(seq_lens_new)
+    fl = 2 * len(seq_lens_new) * c["width"] * c["vocab"] + 2 * n * 2 * c["width"] ** 2 * c["loop"]["times"]
+    for L in _salivik_runs(c):
+        fl += 2 * n * _salivik_layer_params(c, L, L["mlp"]["router"]["top"])
+        m = L["mixer"]
+        if L["type"] == "retention":
+            fl += 4 * n * m["heads"] * m["dim"] * m["vdim"]
+            continue
+        pairs = sum(sum(min(i + 1, m["mask"]["size"]) for i in range(t)) for t in seq_lens_new)
+        if L["type"] == "latent_attention":
+            fl += 2 * pairs * m["heads"] * (2 * m["kv_rank"] + m["rot_dim"])
+        else:
+            fl += 2 * pairs * m["heads"] * 2 * m["dim"]
+    return fl
+
+
+def salivik_compare(args):
+    """Decode and prefill of Salivik beside Pedatar (the closest of the engine's models: latent attention, a mixer with a
+    state per request, routed experts beside a shared one, root-mean-square norms) at the layer sizes of GPT-2 124M and
+    355M; one JSON line."""
+    import numpy as np
+    el, dkey = 2, "bf16"
+    out = {"metric": "decode tok/s at batch 8 of Salivik at GPT-2 124M layer sizes (beside Pedatar at the same sizes: see points)",
+           "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": dkey, "steps": args.steps, "warmup": args.warmup,
+           "data": "synthetic (random weights drawn on the GPU, uniform-random token ids)", "points": {}, "points_frac": {}}
+    for size in ("124m", "355m"):
+        for design in ("pedatar", "salivik"):
+            rng = np.random.default_rng(0)
+            cfg = pedatar_config(size) if design == "pedatar" else salivik_config(size)
+            nbytes = pedatar_step_bytes if design == "pedatar" else salivik_step_bytes
+            model = engine_from_gpu_weights(cfg, "bfloat16", 64, kernels=args.kernels)
+            key = f"{design}_{size}"
+            for b in (1, 8, 64):
+                steps = min(args.steps, 128)
+                d, cm = decode_run(model, cfg, rng, b, args.prompt_len, steps, 8)
+                out["points"][f"{key}_decode_b{b}"] = round(b * steps / d, 1)
+                out["points_frac"][f"{key}_decode_b{b}"] = round(nbytes(cfg, el, b, cm) / (d / steps) / 1e9 / HBM_GBS, 4)
+            fl = pedatar_step_flops(cfg, [1024, 1024]) if design == "pedatar" else salivik_step_flops(cfg, [1024, 1024])
+            pf = prefill_run(model, cfg, rng, dkey, flops=fl)
+            out["points"][f"{key}_prefill_2048"] = pf["value"]
+            out["points_frac"][f"{key}_prefill_2048"] = pf["frac"]
+            if args.profile_stages:
+                print(f"==== {key}", file=sys.stderr)
+                kernel_table(model, cfg, rng, args.batch, args.prompt_len)
+            del model
+    out["value"] = out["points"]["salivik_124m_decode_b8"]
+    out["config"] = {"model": "salivik beside pedatar at gpt2-124m and gpt2-355m layer sizes", "global_batch": 8,
+                     "prompt_len": args.prompt_len,
+                     "salivik": "latent attention (as Pedatar's, with a window of 512, a sink and ramped speeds), attention "
+                                "whose keys are its values (GPT-2's heads on a quarter as many key heads, window 512, sink, "
+                                "output gate) and retention (GPT-2's heads, 64 x 64 states) in turn; 8 capped gated experts of "
+                                "2/3 width (2 a token) beside a shared one of 4/3 width; the first three layers run twice",
+                     "parallelism": "single-gpu"}
+    print(json.dumps(out))
+    return 0
+
+
 def design_compare(args):
     """Decode and prefill of another design beside its like at equal sizes; one JSON line."""
     if args.design == "pedatar":
         return pedatar_compare(args)
     if args.design == "pafolorn":
         return pafolorn_compare(args)
+    if args.design == "salivik":
+        return salivik_compare(args)
     return virudra_compare(args)
 
 
@@ -552,10 +677,11 @@ def main():
     ap.add_argument("--pool-tokens", type=int, default=None,
                     help="mixed workload: tokens of cache the pool holds (default: every request at full length; fewer force "
                          "requests out of the cache and back, which the line reports as preemptions)")
-    ap.add_argument("--design", default="gpt2", choices=["gpt2", "virudra", "pedatar", "pafolorn"],
+    ap.add_argument("--design", default="gpt2", choices=["gpt2", "virudra", "pedatar", "pafolorn", "salivik"],
                     help="virudra: that design beside GPT-2 at equal sizes (decode at batch 1, 8, 64 and the prefill of 2,048 "
                          "tokens, at 124M and 355M layer sizes) instead of the default workload; pedatar: that design beside "
-                         "Virudra, likewise; pafolorn: that design beside Pedatar, likewise")
+                         "Virudra, likewise; pafolorn: that design beside Pedatar, likewise; "
+                         "salivik: that design beside Pedatar, likewise")
     ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
                     help="mixed: only the mixed workload, on --model (64 requests with prompts of 16 to 895 tokens arrive at "
                          "once, prompt portions of 512 tokens run beside the decoding of the others, 128 new tokens each)")
@@ -567,7 +693,7 @@ def main():
     import numpy as np
     from deliverance_amd.random_model import random_model
 
-    if args.design in ("virudra", "pedatar", "pafolorn"):
+    if args.design in ("virudra", "pedatar", "pafolorn", "salivik"):
         return design_compare(args)
     cfg = model_config(args.model, args.layers, args.n_positions)
     full_layers = MODELS[args.model]["n_layer"]

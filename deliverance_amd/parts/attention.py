@@ -147,11 +147,21 @@ class CausalSelfAttention(Mixer):
         N = x.shape[0]
         ln = norm.fusable_params()
         rms = getattr(norm, "rms_params", lambda: None)() if ln is None else None
-        if (ln is None and rms is None) or not self._epilogue_write() or not ops.can_fuse_ln(N, x, self.qkv_weight):
+        if (ln is None and rms is None) or self.qk_norm is not None or not ops.can_fuse_ln(N, x, self.qkv_weight):
             return False
-        qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
         slot = ctx.cache.kv[call.cache]
         group = ctx.group_of(call.cache)
+        if not self._epilogue_write():
+            # the norm and the one product in one kernel; the turn of q and k and the cache write follow
+            qkv = ctx.buf("qkv", N, self.proj_cols, ctx.dtype)
+            if ln is not None:
+                ops.linear_ln(x, None, N, ln[0], ln[1], ln[2], self.qkv_weight, self.qkv_bias, qkv)
+            else:
+                ops.linear_rms(x, None, N, rms[0], rms[1], rms[2], self.qkv_weight, self.qkv_bias, qkv)
+            self._turn_and_keep(ctx, qkv, slot, group, call)
+            self._attend(ctx, qkv, x if into is None else into, slot, group, call)
+            return True
+        qkv = ctx.buf("qkv", N, self.qkv_cols, ctx.dtype)
         kv = dict(kv_cache=slot if call.write else None, slot_map=ctx.slot_maps[group] if call.write else None,
                   q_cols=self.q_cols)
         if ln is not None:
@@ -190,15 +200,19 @@ class CausalSelfAttention(Mixer):
                              ctx.cache.page_size)
         else:
             ops.linear(h, self.qkv_weight, self.qkv_bias, qkv)
-            if self.position is not None:
-                self.position.apply_qk(ctx, qkv, self.n_heads, self.n_kv_heads, self.head_dim)
-            if call.write and self.v_head_dim == self.head_dim:
-                ops.kv_write(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
-                             self.n_kv_heads, self.head_dim)
-            elif call.write:
-                ops.kv_write_split(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
-                                   self.n_kv_heads, self.head_dim, self.v_head_dim, ctx.cache.page_size)
+            self._turn_and_keep(ctx, qkv, slot, group, call)
         self._attend(ctx, qkv, x, slot, group, call)
+
+    def _turn_and_keep(self, ctx: StepContext, qkv: torch.Tensor, slot: torch.Tensor, group: int, call) -> None:
+        """The position encoding of q and k in place, then keys and values into the cache."""
+        if self.position is not None:
+            self.position.apply_qk(ctx, qkv, self.n_heads, self.n_kv_heads, self.head_dim)
+        if call.write and self.v_head_dim == self.head_dim:
+            ops.kv_write(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
+                         self.n_kv_heads, self.head_dim)
+        elif call.write:
+            ops.kv_write_split(qkv, self.q_cols, self.q_cols + self.kv_cols, slot, ctx.slot_maps[group],
+                               self.n_kv_heads, self.head_dim, self.v_head_dim, ctx.cache.page_size)
 
     def _attend(self, ctx: StepContext, qkv: torch.Tensor, x: torch.Tensor, slot: torch.Tensor, group: int,
                 call) -> None:

@@ -75,11 +75,10 @@ class RotaryPositions(PositionEncoding):
                           self.dims, self.interleaved, self.magnitude)
 
     def apply_qk(self, ctx, qkv, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
-        """Queries and keys of a fused q | k | v row, in place."""
-        q = qkv[:, :n_heads * head_dim]
-        k = qkv[:, n_heads * head_dim:(n_heads + n_kv_heads) * head_dim]
-        self.apply(ctx, q, q, n_heads, head_dim, head_dim, head_dim)
-        self.apply(ctx, k, k, n_kv_heads, head_dim, head_dim, head_dim)
+        """Queries and keys of a fused q | k | v row, in place: they lie side by side as heads of one size, so one
+        launch turns both."""
+        qk = qkv[:, :(n_heads + n_kv_heads) * head_dim]
+        self.apply(ctx, qk, qk, n_heads + n_kv_heads, head_dim, head_dim, head_dim)
 
 
 register_position("rotary", RotaryPositions)

@@ -59,11 +59,28 @@ class Retention(Mixer):
     def cache_need(self):
         return StateNeed(self.H * self.Dv * self.D)
 
-    def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
-        N, H = h.shape[0], self.H
-        state = ctx.cache.state[call.cache]
+    normed_into = True
+
+    def forward_normed(self, ctx: StepContext, norm, x: torch.Tensor, call, into=None) -> bool:
+        """Small steps: the root-mean-square norm in front and the one product in one kernel."""
+        N = x.shape[0]
+        rms = getattr(norm, "rms_params", lambda: None)()
+        if rms is None or not ops.can_fuse_ln(N, x, self.in_weight):
+            return False
+        gain, offset, eps = rms
         proj = ctx.buf("retention_in", N, self.in_weight.shape[0], ctx.dtype)
+        ops.linear_rms(x, None, N, gain, offset, eps, self.in_weight, None, proj)
+        self._mix(ctx, proj, x if into is None else into, call)
+        return True
+
+    def forward(self, ctx: StepContext, h: torch.Tensor, x: torch.Tensor, call) -> None:
+        proj = ctx.buf("retention_in", h.shape[0], self.in_weight.shape[0], ctx.dtype)
         ops.linear(h, self.in_weight, None, proj)
+        self._mix(ctx, proj, x, call)
+
+    def _mix(self, ctx: StepContext, proj: torch.Tensor, x: torch.Tensor, call) -> None:
+        N, H = proj.shape[0], self.H
+        state = ctx.cache.state[call.cache]
         if self.rotary is not None and self.rotary.dims:
             qk = proj[:, :2 * self.qk_cols]                 # q and k are 2 H heads side by side: one launch, in place
             self.rotary.apply(ctx, qk, qk, 2 * H, self.D, self.D, self.D)

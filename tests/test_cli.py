@@ -71,6 +71,21 @@ def test_random_then_inspect_a_design_with_parallel_mixers(tmp_path):
     assert "l0.mix.left.q.norm" in p.stdout and "l0.mix.right.A_log" in p.stdout and "l0.ls1" in p.stdout and "embed.norm" in p.stdout
 
 
+def test_random_then_inspect_a_design_with_a_loop_of_layers(tmp_path):
+    """... and on a Salivik configuration: a looped layer stores its tensors once and keeps a cache slot a pass."""
+    from salivik_models import CONFIG_S
+    cfg = tmp_path / "config.json"
+    cfg.write_text(json.dumps(CONFIG_S))
+    out = tmp_path / "model"
+    p = run("random", "--config", str(cfg), "--seed", "6", "--out", str(out))
+    assert p.returncode == 0, p.stderr
+    p = run("inspect", str(out))
+    assert p.returncode == 0, p.stderr
+    assert "architecture Salivik: 4 layers, width 64, vocabulary 300" in p.stdout and "8 layer calls, 8 cache slots" in p.stdout
+    assert "loop.in" in p.stdout and "l1.mix.sink" in p.stdout and "l2.mix.g" in p.stdout and "l1.mlp.router.b" in p.stdout
+    assert "l0.mix.v" in p.stdout and "l2.mix.v" not in p.stdout and "embed.norm" in p.stdout
+
+
 def test_help_names_the_reference_options():
     p = run("generate", "--help")
     for opt in ("--model", "--working-dtype", "--max-tokens", "--temperature", "--seed", "--warmup-cases", "--max-cases",

@@ -1,0 +1,171 @@
+"""Salivik without a GPU: its configuration, run order and loop, tensor declarations, the random-weights mode, what
+its mixers ask of the cache, and the plain implementation against other ways of writing the same formulas."""
+import json
+
+import numpy as np
+import pytest
+import torch
+
+import plain_salivik as P
+from salivik_models import CONFIG_S, CONFIG_T, CONFIG_U
+
+
+def test_config_reads_every_size_and_constant():
+    from deliverance_amd.config import ConfigError, SalivikConfig
+    from deliverance_amd.config.specs import (AttentionSpec, ExpertsFeedForwardSpec, GatedFeedForwardSpec, LatentAttentionSpec,
+                                              RetentionSpec)
+    for cfg in (CONFIG_S, CONFIG_T, CONFIG_U):
+        mc = SalivikConfig.from_dict(cfg).to_model_config()
+        assert (mc.vocab_size, mc.width) == (cfg["vocab"], cfg["width"])
+        for n in (mc.final_norm, mc.embed_norm):
+            assert n.kind == "rmsnorm" and n.gain_offset == 0.0 and n.eps == cfg["norm"]["eps"]
+        assert not mc.tie_word_embeddings and mc.embed_position.kind == "none" and mc.input_mix == ("loop" in cfg)
+        for spec, raw in zip(mc.layers, cfg["layers"]):
+            m, a = raw["mixer"], spec.mixer
+            assert spec.pre_mixer_norm is not None and spec.post_mixer_norm is None and spec.post_ff_norm is None
+            if raw["type"] == "attention":
+                assert isinstance(a, AttentionSpec) and a.values_are_keys and a.sink == "zero" and a.out_gate == "sigmoid"
+                assert (a.n_heads, a.n_kv_heads, a.head_dim, a.value_dim, a.scale, a.window) == \
+                    (m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"], m["mask"]["size"])
+                assert (a.position.dims, a.position.base, a.position.interleaved) == (m["rot"]["dims"], m["rot"]["base"], False)
+                assert not a.qkv_bias and not a.out_bias and a.keep_first == 0
+            elif raw["type"] == "retention":
+                assert isinstance(a, RetentionSpec)
+                assert (a.n_heads, a.head_dim, a.v_head_dim, list(a.decay), a.norm_eps) == \
+                    (m["heads"], m["dim"], m["vdim"], m["decay"], cfg["norm"]["eps"])
+                assert (a.rotary.dims, a.rotary.base, a.rotary.interleaved) == (m["rot"]["dims"], m["rot"]["base"], False)
+            else:
+                assert isinstance(a, LatentAttentionSpec) and a.sink
+                assert (a.n_heads, a.head_dim, a.rot_dim, a.v_head_dim, a.q_rank, a.kv_rank, a.scale, a.window) == \
+                    (m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["q_rank"], m["kv_rank"], m["scale"], m["mask"]["size"])
+                sc = m["rot"].get("scaling")
+                assert (a.rotary.scaling is None) == (sc is None) and not a.rotary.interleaved
+                if sc:
+                    assert (a.rotary.scaling.factor, a.rotary.scaling.original, a.rotary.scaling.fast, a.rotary.scaling.slow) == \
+                        (sc["factor"], sc["original"], sc["fast"], sc["slow"])
+            f, rf = spec.feed_forward, raw["mlp"]
+            if rf is None:
+                assert f is None and spec.pre_ff_norm is None
+            elif rf["kind"] == "dense":
+                assert isinstance(f, GatedFeedForwardSpec) and (f.inner, f.limit, f.activation) == (rf["ff"], rf["limit"], "glu_capped")
+            else:
+                assert isinstance(f, ExpertsFeedForwardSpec) and f.router == "softmax_top" and f.gated and f.router_bias
+                assert (f.inner, f.limit, f.n_experts, f.top) == (rf["expert"]["ff"], rf["expert"]["limit"], rf["router"]["experts"], rf["router"]["top"])
+                assert (f.shared_inner, f.shared_limit) == ((rf["shared"]["ff"], rf["shared"]["limit"]) if rf["shared"] else (0, 0.0))
+        assert SalivikConfig.from_dict(mc.raw).to_model_config() == mc           # what is written out reads back the same
+    # what is missing is named, all of it at once
+    broken = json.loads(json.dumps(CONFIG_S))
+    del broken["norm"]["eps"], broken["layers"][1]["mixer"]["rot"]["scaling"]["fast"], broken["layers"][0]["mixer"]["decay"]
+    del broken["layers"][2]["mlp"]["router"]["top"], broken["layers"][2]["mixer"]["mask"], broken["loop"]["times"]
+    del broken["layers"][1]["mlp"]["shared"]["limit"], broken["layers"][0]["mlp"]["limit"]
+    with pytest.raises(ConfigError) as e:
+        SalivikConfig.from_dict(broken)
+    for key in ("norm.eps", "layers[1].mixer.rot.scaling.fast", "layers[0].mixer.decay", "layers[2].mlp.router.top",
+                "layers[2].mixer.mask", "loop.times", "layers[1].mlp.shared.limit", "layers[0].mlp.limit"):
+        assert key in str(e.value)
+    for change, match in ((lambda c: c["layers"][0].update(type="mamba1"), "mamba1"),
+                          (lambda c: c["layers"][2]["mixer"]["rot"].update(dims=7), "rot.dims"),
+                          (lambda c: c["layers"][2]["mixer"].update(kv_heads=3), "key heads"),
+                          (lambda c: c["layers"][2]["mixer"].update(vdim=8), "vdim"),
+                          (lambda c: c["layers"][0]["mixer"].update(decay=[0.5]), "decays"),
+                          (lambda c: c["loop"].update(stop=9), "loop"),
+                          (lambda c: c["layers"][1]["mlp"]["router"].update(top=9), "top")):
+        other = json.loads(json.dumps(CONFIG_S))
+        change(other)
+        with pytest.raises(ConfigError, match=match):
+            SalivikConfig.from_dict(other)
+
+
+def test_every_pass_of_a_loop_keeps_a_cache_of_its_own_and_starts_by_mixing():
+    from deliverance_amd.config import SalivikConfig
+    mc = SalivikConfig.from_dict(CONFIG_S).to_model_config()
+    assert [(c.layer, c.cache, c.mix_input) for c in mc.schedule] == \
+        [(0, 0, False), (1, 1, True), (2, 2, False), (1, 3, True), (2, 4, False), (1, 5, True), (2, 6, False), (3, 7, False)]
+    assert mc.n_cache_slots == 8
+    assert [(i, s) for i, s in P.run_order(CONFIG_S)] == [(c.layer, c.mix_input) for c in mc.schedule]
+    mc = SalivikConfig.from_dict(CONFIG_T).to_model_config()
+    assert [(c.layer, c.cache, c.mix_input) for c in mc.schedule] == [(0, 0, False), (1, 1, False), (2, 2, False)] and not mc.input_mix
+    mc = SalivikConfig.from_dict(CONFIG_U).to_model_config()             # a loop of one pass still mixes once
+    assert [(c.layer, c.cache, c.mix_input) for c in mc.schedule] == [(0, 0, True), (1, 1, False), (2, 2, False)] and mc.input_mix
+
+
+def test_tensors_and_what_the_mixers_keep(tmp_path):
+    from deliverance_amd import models  # noqa: F401
+    from deliverance_amd.parts import KVNeed, StateNeed
+    from deliverance_amd.random_model import random_model
+    from deliverance_amd.registry import ModelSupport
+    from deliverance_amd.weights.loader import load_declared
+    arch = ModelSupport.detect(CONFIG_S)
+    assert arch.name == "Salivik"
+    mc = arch.read_config(CONFIG_S)
+    names = {d.name: tuple(d.shape) for d in arch.declare_tensors(mc)}
+    E = CONFIG_S["width"]
+    assert names["loop.in"] == (E, 2 * E) and names["embed.norm"] == (E,) and names["head"] == (CONFIG_S["vocab"], E)
+    assert names["l2.mix.k"] == (2 * 16, E) and names["l2.mix.g"] == (4 * 16, E) and "l2.mix.v" not in names
+    assert names["l0.mix.v"] == (2 * 24, E) and names["l0.mix.q"] == (2 * 16, E) and names["l0.mlp.gate"] == (96, E)
+    assert names["l1.mix.sink"] == (2,) and names["l1.mix.dkv"] == (40 + 8, E) and names["l1.mix.uq"] == (2 * (16 + 8), 24)
+    assert names["l1.mlp.router.b"] == (4,) and names["l1.mlp.e3.up"] == (32, E) and names["l1.mlp.shared.down"] == (E, 48)
+    assert "l3.norm2" not in names and not any(n.startswith("l4.") for n in names)
+    assert "loop.in" not in {d.name for d in arch.declare_tensors(arch.read_config(CONFIG_T))}
+    random_model(str(tmp_path), CONFIG_S, 3)
+    t = load_declared(str(tmp_path), arch.declare_tensors(mc))
+    from deliverance_amd.models.causal_lm import CausalLM
+    from deliverance_amd.kernels import build
+    if build.library_path() is None:
+        pytest.skip("the kernel library is not built")
+    model = CausalLM(mc, arch.bind_tensors(mc, t), torch.float32, "cpu")
+    needs = model.cache_needs()
+    assert needs[0] == StateNeed(2 * 24 * 16) and needs[7] == StateNeed(1 * 16 * 32)
+    for slot in (1, 3, 5):
+        assert needs[slot] == KVNeed(1, 40 + 8, 24, 40, values_in_keys=True)
+    for slot in (2, 4, 6):
+        assert needs[slot] == KVNeed(2, 16, 40, None)
+
+
+def test_the_plain_model_written_another_way():
+    """Retention as a sum over earlier tokens with powers of the decay; the softmax's extra term as one more key whose
+    score is the sink and whose value is zero; the ramped speeds at their two ends."""
+    rng = np.random.default_rng(0)
+    T, E = 23, 16
+    m = {"heads": 2, "dim": 8, "vdim": 4, "decay": [0.9, 0.5], "rot": {"base": 100.0, "dims": 4}}
+    W = {"mix.q": rng.normal(size=(16, E)), "mix.k": rng.normal(size=(16, E)), "mix.v": rng.normal(size=(8, E)),
+         "mix.g": rng.normal(size=(8, E)), "mix.o": rng.normal(size=(E, 8))}
+    h = rng.normal(size=(T, E))
+    got = P.retention(W, "", m, h, 1e-5)
+    q = P.turn_halves((h @ W["mix.q"].T).reshape(T, 2, 8), np.arange(T), m["rot"])
+    k = P.turn_halves((h @ W["mix.k"].T).reshape(T, 2, 8), np.arange(T), m["rot"]) / np.sqrt(8.0)
+    v = (h @ W["mix.v"].T).reshape(T, 2, 4)
+    o = np.zeros((T, 2, 4))
+    for hd in range(2):
+        for t in range(T):
+            for s in range(t + 1):
+                o[t, hd] += m["decay"][hd] ** (t - s) * (q[t, hd] @ k[s, hd]) * v[s, hd]
+    o = o / np.sqrt((o ** 2).mean(-1, keepdims=True) + 1e-5)
+    want = (o.reshape(T, 8) * P.swish(h @ W["mix.g"].T)) @ W["mix.o"].T
+    assert np.abs(got - want).max() <= 1e-9 * np.abs(want).max()
+    # the extra term as a key of its own
+    s = rng.normal(size=(5, 7))
+    mask = rng.random((5, 7)) < 0.7
+    mask[:, 0] = True
+    sink = rng.normal(size=(5, 1))
+    w = P.softmax_with_sink(s, mask, sink)
+    full = np.concatenate([np.where(mask, s, -np.inf), sink], axis=1)
+    e = np.exp(full - full.max(-1, keepdims=True))
+    assert np.abs(w - (e / e.sum(-1, keepdims=True))[:, :7]).max() <= 1e-12
+    # pairs that turn fast keep their speed, the slowest turn `factor` times slower; sine and cosine grow
+    r = {"base": 10000.0, "dims": 32, "scaling": {"factor": 4.0, "original": 256, "fast": 16.0, "slow": 1.0}}
+    plain, _ = P.turn_speeds({"base": 10000.0, "dims": 32})
+    speeds, length = P.turn_speeds(r)
+    assert speeds[0] == plain[0] and abs(speeds[-1] - plain[-1] / 4.0) <= 1e-15 and abs(length - (0.1 * np.log(4.0) + 1.0)) <= 1e-15
+    assert all(plain[i] / 4.0 - 1e-15 <= speeds[i] <= plain[i] + 1e-15 for i in range(16))
+
+
+def test_the_engines_speeds_are_the_plain_ones():
+    from deliverance_amd.config.specs import RampedSpeedsSpec
+    from deliverance_amd.parts.positions import ramped_speeds
+    for dims, base, sc in ((16, 1e6, (2.0, 1024, 32.0, 1.0)), (32, 10000.0, (4.0, 256, 16.0, 1.0)), (8, 100.0, (1.0, 32, 4.0, 2.0)),
+                           (24, 500.0, (16.0, 32, 4.0, 0.5))):
+        plain = [base ** (-2.0 * i / dims) for i in range(dims // 2)]
+        got, mag = ramped_speeds(plain, dims, base, RampedSpeedsSpec(*sc))
+        want, length = P.turn_speeds({"base": base, "dims": dims, "scaling": dict(zip(("factor", "original", "fast", "slow"), sc))})
+        assert np.abs(np.asarray(got) - want).max() <= 1e-15 and abs(mag - length) <= 1e-15

@@ -46,6 +46,11 @@ RUNS = {
     "pafolorn": ["tests/test_pafolorn_gpu.py", "-n", "4"] if FULL else
                 ["tests/test_pafolorn_gpu.py", "-n", "3", "-m", QUICK, "-k",
                  "not token_by_token and not (mixed_batches and (F or G)) and not (portions and sizes0)"],
+    # a fifth design's kernels and parts (retention, attention whose keys are its values with a term without a key and
+    # an output gate, latent attention with a window and a learned sink, capped gated feed-forwards, a router that
+    # weighs the chosen logits among themselves) and its models through the step function
+    "salivik": ["tests/test_salivik_gpu.py", "-n", "4"] if FULL else
+               ["tests/test_salivik_gpu.py", "-n", "3", "-m", QUICK, "-k", "not (portions and sizes0)"],
     "replay": ["tests/test_replay_gpu.py", "-n", "4"] if FULL else
               ["tests/test_replay_gpu.py", "-n", "2", "-k", "(mixed and (A or B) and not 32) or want_subset or errors_leave or first_tokens"],
     # inner sizes of 32 in an engine step: qkv and fc of seed 11 (and, in the full run, proj of seed 5)
