@@ -6,11 +6,14 @@
 // q and k come turned by their positions already; k is multiplied by k_scale here (D^-1/2).
 //
 // The columns of S do not meet: column c needs q, k and v[c] only.  A column is shared out over 16 neighbouring
-// lanes, lane j holding rows j, j + 16, ... in registers; the sum over rows is taken inside the lane and then over
+// lanes, lane j holding the RPL consecutive rows from j * RPL on in registers (so that a token's q and k entries are
+// one 16-byte LDS read each where RPL is a multiple of 4); the sum over rows is taken inside the lane and then over
 // the 16 lanes by DPP additions.  A wavefront holds 4 columns, a workgroup of 4 wavefronts 16; the grid is
 // (column blocks x heads x sequences), each walking its sequence's portion in order.  Tokens come through LDS in
-// blocks of 16: every thread asks for its share of the next block (RPL entries of q and of k, one of v) before it
-// walks the block at hand, so that the walk hides the trip to memory.  A token's result is the same bits however the
+// blocks of TB (64 for key sizes up to 64, 32 up to 128, else 16: 32 KB of LDS): every thread asks for its share of
+// the next block before it walks the block at hand, and a block's walk (about 3 us) is longer than the trip to
+// memory.  Inside a block the walk goes in groups of 16 tokens of straight-line code; lane j keeps the result of a
+// group's token j, so a group's results leave in one store a lane.  A token's result is the same bits however the
 // sequence was cut into steps and whatever else the step holds: the walk is the recurrence itself, and the order of
 // the sum over rows depends on D only.
 //
@@ -20,7 +23,7 @@
 
 #define RET_LPC 16            // lanes that share a column
 #define RET_CPB 16            // columns of a workgroup
-#define RET_TB 16             // tokens of a block
+#define RET_GROUP 16          // tokens whose results the 16 lanes of a column keep, one each
 #define RET_MAX_D 256
 
 struct RetArgs {
@@ -39,7 +42,10 @@ template <typename T, int RPL>
 __global__ void __launch_bounds__(RET_CPB * RET_LPC)
 retention_kernel(RetArgs A) {
   constexpr int DP = RPL * RET_LPC;                 // D rounded up to what the lanes hold
-  __shared__ float qs[RET_TB][DP], ks[RET_TB][DP], vs[RET_TB][RET_CPB];
+  constexpr int TB = RPL <= 4 ? 64 : (RPL <= 8 ? 32 : 16);       // tokens of a block
+  constexpr int PER = TB * RPL / RET_LPC;           // entries of q (and of k) of a block that a thread brings
+  constexpr int PERV = TB / RET_GROUP;              // ... and of v
+  __shared__ __attribute__((aligned(16))) float qs[TB][DP], ks[TB][DP], vs[TB][RET_CPB];
   const int t = threadIdx.x, j = t % RET_LPC, c = t / RET_LPC;
   const int h = blockIdx.y, s = blockIdx.z;
   const int col = blockIdx.x * RET_CPB + c;
@@ -54,66 +60,85 @@ retention_kernel(RetArgs A) {
   float* srow = (slot >= 0 && col_ok) ? A.state + (size_t)slot * A.state_ld + ((size_t)h * A.Dv + col) * A.D : nullptr;
 #pragma unroll
   for (int i = 0; i < RPL; ++i) {
-    const int r = j + RET_LPC * i;
+    const int r = j * RPL + i;
     S[i] = (srow && r < A.D) ? srow[r] : 0.f;
   }
 
-  // this thread's share of a block: entries t + 256 i of [token][DP] for q and for k, entry t of [token][16] for v
-  T rq[RPL], rk[RPL], rv;
-  unsigned ok = 0;                                  // bit i: entry i exists; bit 31: the value entry exists
+  // this thread's share of a block: entries t + 256 i of [token][DP] for q and for k, of [token][16] for v
+  T rq[PER], rk[PER], rv[PERV];
+  unsigned long long ok = 0;                        // bit i: entry i of q and k exists; bit 60 + i: entry i of v
   auto fetch = [&](int t0) {
     ok = 0;
 #pragma unroll
-    for (int i = 0; i < RPL; ++i) {
+    for (int i = 0; i < PER; ++i) {
       const int idx = t + 256 * i, tok = idx / DP, r = idx % DP;
       const bool e = t0 + tok < n_tok && r < A.D;
       const size_t at = (size_t)(row0 + (e ? t0 + tok : 0)) * A.ld + (size_t)h * A.D + (e ? r : 0);
       rq[i] = base[at + A.q_off];                   // (unconditional, from a place that exists; looked at when parked)
       rk[i] = base[at + A.k_off];
-      ok |= (unsigned)e << i;
+      ok |= (unsigned long long)e << i;
     }
-    const int tok = t / RET_CPB, cc = blockIdx.x * RET_CPB + t % RET_CPB;
-    const bool e = t0 + tok < n_tok && cc < A.Dv;
-    rv = base[(size_t)(row0 + (e ? t0 + tok : 0)) * A.ld + A.v_off + (size_t)h * A.Dv + (e ? cc : 0)];
-    ok |= (unsigned)e << 31;
-  };
-  auto park = [&]() {
 #pragma unroll
-    for (int i = 0; i < RPL; ++i) {
+    for (int i = 0; i < PERV; ++i) {
+      const int idx = t + 256 * i, tok = idx / RET_CPB, cc = blockIdx.x * RET_CPB + idx % RET_CPB;
+      const bool e = t0 + tok < n_tok && cc < A.Dv;
+      rv[i] = base[(size_t)(row0 + (e ? t0 + tok : 0)) * A.ld + A.v_off + (size_t)h * A.Dv + (e ? cc : 0)];
+      ok |= (unsigned long long)e << (60 + i);
+    }
+  };
+  auto park = [&](int nt) {                         // (tokens past the block's last are never read)
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
       const int idx = t + 256 * i, tok = idx / DP, r = idx % DP;
       const bool e = (ok >> i) & 1u;
-      qs[tok][r] = e ? to_f32(rq[i]) : 0.f;
-      ks[tok][r] = e ? to_f32(rk[i]) * A.k_scale : 0.f;
+      if (tok < nt) {
+        qs[tok][r] = e ? to_f32(rq[i]) : 0.f;
+        ks[tok][r] = e ? to_f32(rk[i]) * A.k_scale : 0.f;
+      }
     }
-    vs[t / RET_CPB][t % RET_CPB] = (ok >> 31) ? to_f32(rv) : 0.f;
+#pragma unroll
+    for (int i = 0; i < PERV; ++i) {
+      const int idx = t + 256 * i;
+      if (idx / RET_CPB < nt) vs[idx / RET_CPB][idx % RET_CPB] = ((ok >> (60 + i)) & 1u) ? to_f32(rv[i]) : 0.f;
+    }
   };
 
   fetch(0);
-  for (int t0 = 0; t0 < n_tok; t0 += RET_TB) {
+  for (int t0 = 0; t0 < n_tok; t0 += TB) {
+    const int nt = n_tok - t0 < TB ? n_tok - t0 : TB;
     __syncthreads();                                // the block before has been walked by everyone
-    park();
+    park(nt);
     __syncthreads();
-    if (t0 + RET_TB < n_tok) fetch(t0 + RET_TB);
-    const int nt = n_tok - t0 < RET_TB ? n_tok - t0 : RET_TB;
-    float mine = 0.f;                               // lane j keeps the result of the block's token j
-    for (int tk = 0; tk < nt; ++tk) {
-      const float vv = vs[tk][c];
-      float acc = 0.f;
+    if (t0 + TB < n_tok) fetch(t0 + TB);
+    for (int g0 = 0; g0 < nt; g0 += RET_GROUP) {
+      const int ng = nt - g0 < RET_GROUP ? nt - g0 : RET_GROUP;
+      float mine = 0.f;                             // lane j keeps the result of the group's token j
+      auto token = [&](int k) {
+        const int tk = g0 + k;
+        const float vv = vs[tk][c];
+        float acc = 0.f;
 #pragma unroll
-      for (int i = 0; i < RPL; ++i) {
-        const int r = j + RET_LPC * i;
-        S[i] = fmaf(g, S[i], ks[tk][r] * vv);
-        acc = fmaf(S[i], qs[tk][r], acc);
+        for (int i = 0; i < RPL; ++i) {
+          const int r = j * RPL + i;
+          S[i] = fmaf(g, S[i], ks[tk][r] * vv);
+          acc = fmaf(S[i], qs[tk][r], acc);
+        }
+        acc = group_sum<RET_LPC>(acc);
+        mine = k == j ? acc : mine;
+      };
+      if (ng == RET_GROUP) {                        // a whole group: straight-line code, the LDS reads run ahead
+#pragma unroll
+        for (int k = 0; k < RET_GROUP; ++k) token(k);
+      } else {
+        for (int k = 0; k < ng; ++k) token(k);
       }
-      acc = group_sum<RET_LPC>(acc);
-      if (tk == j) mine = acc;
+      if (j < ng && col_ok) A.o[(size_t)(row0 + t0 + g0 + j) * A.o_ld + (size_t)h * A.Dv + col] = mine;
     }
-    if (j < nt && col_ok) A.o[(size_t)(row0 + t0 + j) * A.o_ld + (size_t)h * A.Dv + col] = mine;
   }
   if (A.write && srow) {
 #pragma unroll
     for (int i = 0; i < RPL; ++i) {
-      const int r = j + RET_LPC * i;
+      const int r = j * RPL + i;
       if (r < A.D) srow[r] = S[i];
     }
   }
