@@ -112,7 +112,8 @@ _ARGTYPES = {
     "da_kv_write_split": [_VP, _I, _I, _I, _I, _VP, _VP, _I, _I, _I, _I, _I, _VP],
     "da_gated_act": [_VP, _I, _I, _VP, _I, _I, _I, _I, _F, _VP],
     "da_concat_rows": [_VP, _VP, _I, _I, _I, _I, _I, _VP],
-    "da_retention": [_VP, _I, _I, _I, _I, _I, _VP, _F, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _VP],
+    "da_retention": [_VP, _I, _I, _I, _I, _I, _VP, _F, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _VP,
+                     ctypes.c_long, _VP],
     "da_moe_top": [_VP, _I, _VP, _I, _I, _I, _I, _I, _I, _VP, _VP, _VP],
     "da_softcap": [_VP, ctypes.c_long, _F, _VP],
     "da_moe_route": [_VP, _VP, _I, _VP, _I, _I, _I, _I, _VP, _VP, _VP, _I, _I, _VP, _VP, _VP],
@@ -1450,12 +1451,16 @@ def paged_attention_latent(ctx, q: torch.Tensor, cache_slot: torch.Tensor, group
 
 # ------------------------------------------------------------------------------- retention
 RETENTION_MAX_DIM = 256      # key entries a head of the retention kernel (csrc/retention.hip)
+RETENTION_CHUNK = 128        # tokens of a chunk when a long portion's walk is cut up
+RETENTION_CHUNK_FROM = 256   # portions from this length on are cut up (bfloat16 serving only)
 
 
 def retention(ctx, qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, decay: torch.Tensor, k_scale: float,
               state: torch.Tensor, o: torch.Tensor, n_heads: int, head_dim: int, v_head_dim: int,
-              write: bool = True) -> torch.Tensor:
+              write: bool = True, chunk: Optional[int] = None) -> torch.Tensor:
     """Per head S <- decay[h] S + k v^T, o = S^T q over every sequence of the step, token by token (csrc/retention.hip).
+    ``chunk``: tokens of the chunks that long portions are walked in, side by side (0: every portion in one piece; None:
+    ``RETENTION_CHUNK`` in bfloat16 serving when the step's longest portion has ``RETENTION_CHUNK_FROM`` rows, else 0).
     ``qkv`` [N, ...] holds the turned q and k (H * D entries each, from columns ``q_off`` and ``k_off``) and v (H * Dv
     from ``v_off``) in the step's dtype; k is multiplied by ``k_scale``; ``decay`` float32 [H]; ``state`` [slots, >= H * Dv
     * D] 32-bit is read at each portion's start and, with ``write``, written at its end; ``o`` [N, H * Dv] 32-bit."""
@@ -1471,11 +1476,20 @@ def retention(ctx, qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, decay:
     _need(decay.dtype == torch.float32 and decay.is_contiguous() and decay.numel() == H, "retention: decay must be float32 [H]")
     _need(ld >= H * Dv * D, "retention: the state row is too short")
     _need(ctx.q_start.numel() >= ctx.n_seqs + 1 and ctx.state_slots.numel() >= ctx.n_seqs, "retention: the step's arrays are too short")
+    longest = int(getattr(ctx, "max_query_len", 0) or 0)
+    if chunk is None:
+        chunk = RETENTION_CHUNK if (_MODE == "tuned" and qkv.dtype == torch.bfloat16 and longest >= RETENTION_CHUNK_FROM) else 0
+    n_chunks, ends = 1, None
+    if chunk:
+        _need(chunk % 16 == 0 and longest > 0, "retention: chunks are multiples of 16 tokens and need the longest portion's length")
+        n_chunks = -(-longest // chunk)
+        ends = ctx.buf("retention_ends", ctx.n_seqs * n_chunks, H * Dv * D, torch.float32)
     nb = N * ((2 * H * D + H * Dv) * qkv.element_size() + H * Dv * 4) + 2 * ctx.n_seqs * H * Dv * D * 4
     with _timed("retention", nb, 4 * N * H * D * Dv, "fp32"):
         _check(_lib().da_retention(_ptr(qkv), _dt(qkv), qkv.stride(0), int(q_off), int(k_off), int(v_off), _ptr(decay),
                                    float(k_scale), _ptr(state), ld, _ptr(ctx.state_slots), _ptr(ctx.q_start), _ptr(o),
-                                   o.stride(0), ctx.n_seqs, H, D, Dv, int(bool(write)), _stream()))
+                                   o.stride(0), ctx.n_seqs, H, D, Dv, int(bool(write)), int(chunk), n_chunks, _ptr(ends),
+                                   0 if ends is None else ends.numel(), _stream()))
     return o
 
 

@@ -422,6 +422,53 @@ def test_retention_remembers_the_first_token(dtype):
     assert b.done == [T]
 
 
+@pytest.mark.parametrize("dtype", ["float32", quick("bfloat16")])
+@pytest.mark.parametrize("chunk", [16, quick(32), 48])
+def test_retention_in_chunks_side_by_side(dtype, chunk):
+    """Long portions are walked in chunks that run side by side, with a carry pass between them: the same results and
+    the same kept states as the walk in one piece, by 32-bit rounding; portions that end inside a chunk, at a chunk's
+    edge, and one-token sequences beside them; states that are kept and states that are not."""
+    from deliverance_amd.kernels import ops
+    rng = np.random.default_rng(chunk)
+    H, D, Dv = 3, 20, 24
+    lens = [70, 1, 33, 2 * chunk, 1]
+    N, S = sum(lens), len(lens)
+    cols = 2 * H * D + H * Dv
+    qkv = dev(bf16(rng.normal(size=(N, cols + 5)) * 0.5), DTYPES[dtype])
+    decay = dev([0.5, 0.96875, 1.0], torch.float32)
+    q_start = np.concatenate([[0], np.cumsum(lens)])
+    state0 = rng.normal(size=(S + 1, H * Dv * D + 3)).astype(np.float32)
+    ctx = SimpleNamespace(q_start=dev(q_start), state_slots=dev([4, 1, -1, 0, 3]), n_seqs=S, max_query_len=max(lens),
+                          buf=lambda name, r, c_, dt: torch.empty(r, c_, dtype=dt, device=DEV))
+    outs = {}
+    for write in (True, False):
+        for ch in (0, chunk):
+            st = dev(state0, torch.float32)
+            o = torch.full((N, H * Dv), float("nan"), dtype=torch.float32, device=DEV)
+            ops.retention(ctx, qkv, 2, 2 + H * D, 2 + 2 * H * D, decay, D ** -0.5, st, o, H, D, Dv, write=write, chunk=ch)
+            outs[(write, ch)] = (host(o), host(st))
+        a, b = outs[(write, 0)], outs[(write, chunk)]
+        assert np.isfinite(b[0]).all()
+        assert np.abs(a[0] - b[0]).max() <= 2e-6 * np.abs(a[0]).max()
+        assert np.abs(a[1] - b[1]).max() <= 2e-6 * np.abs(a[1]).max()
+        if not write:
+            assert np.array_equal(b[1], state0.astype(np.float64))
+    assert np.array_equal(outs[(True, chunk)][1][2], state0[2].astype(np.float64)), "a slot that no sequence has was written"
+    # and the walk in one piece against the formula, from the given states
+    x = host(qkv)[:, 2:2 + cols]
+    want = np.zeros((N, H, Dv))
+    slots = [4, 1, -1, 0, 3]
+    for s_, (a0, a1) in enumerate(zip(q_start[:-1], q_start[1:])):
+        for h_ in range(H):
+            St = np.zeros((D, Dv)) if slots[s_] < 0 else state0[slots[s_], h_ * Dv * D:(h_ + 1) * Dv * D].reshape(Dv, D).T.astype(np.float64)
+            for t in range(a0, a1):
+                q, k = x[t, h_ * D:(h_ + 1) * D], x[t, H * D + h_ * D:H * D + (h_ + 1) * D] * D ** -0.5
+                v = x[t, 2 * H * D + h_ * Dv:2 * H * D + (h_ + 1) * Dv]
+                St = float(host(decay)[h_]) * St + np.outer(k, v)
+                want[t, h_] = St.T @ q
+    assert np.abs(outs[(True, 0)][0] - want.reshape(N, H * Dv)).max() <= 3e-6 * np.abs(want).max()
+
+
 # ------------------------------------------------------------------------------------------ whole models
 @pytest.fixture(scope="module")
 def smodels(tmp_path_factory):
@@ -504,6 +551,26 @@ def test_mixed_batches_over_a_small_pool(smodels, name, dtype):
             one = helpers.replay(alone, helpers.trace_whole(rid, ids))[rid]
             scale = float(np.sqrt((one.astype(np.float64) ** 2).mean()))
             assert np.abs(one.astype(np.float64) - got[rid]).max() <= 2e-5 * scale
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts(smodels, dtype):
+    """Prompts of several hundred tokens at once and in long portions (the forms that kernels keep for long portions),
+    beside a short one; then decoding goes on from what they left."""
+    helpers.skip_in_simulation_if(True)
+    m = smodels["S"]
+    ids, other = m.prompt(700, salt=40), m.prompt(9, salt=41)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": ids[:300], "want": list(range(300))}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": other[:8], "want": list(range(8))},
+                                     {"id": "a", "tokens": ids[300:690], "want": list(range(390))}], "end": []}]
+    for i in range(690, 700):
+        entries = [{"id": "a", "tokens": [ids[i]], "want": [0]}]
+        if i == 690:
+            entries.append({"id": "b", "tokens": [other[8]], "want": [0]})
+        steps.append({"step": len(steps), "entries": entries, "end": ["b"] if i == 690 else []})
+    steps[-1]["end"].append("a")
+    s = helpers.trace_session(m.folder, dtype, 832, poison_freed=True, state_slots=2)
+    run(m, s, steps, [("a", ids), ("b", other)], dtype, "long prompts")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
