@@ -8,6 +8,10 @@
 //                    (i, i + dims / 2): (u, v) -> (u cos a - v sin a, v cos a + u sin a), a = position * speeds[i]
 //                    (speeds in double precision; sine and cosine of the double angle, used in 32-bit)
 //
+// `v_from_k`: the rows hold no values; a key as it was projected (normalised, not turned) is also the value (Dv = D).
+// `pass_cols`: so many columns behind q | k | v of the rows (a gate's, say) go over into the queries' rows behind the
+// queries, converted.  `mag` multiplies sine and cosine (the length that a turned pair gains; 1 as a rule).
+//
 // A page of the cache slot holds Hkv * page * D keys (rows of D), then Hkv * Dv * page values (dimension-major);
 // slot_map[n] = page id * page + row, or -1 for a token whose keys are not kept.  One workgroup a token.
 #include "common.h"
@@ -21,7 +25,8 @@ __global__ void __launch_bounds__(PREP_THREADS)
 attn_prepare_kernel(const float* __restrict__ raw, int ld, int Hq, int Hkv, int D, int Dv, const void* __restrict__ gq,
                     int gq_dtype, const void* __restrict__ gk, int gk_dtype, float eps, int whole,
                     const int* __restrict__ positions, const double* __restrict__ speeds, int dims, int interleaved,
-                    T* __restrict__ q_out, int q_ld, T* __restrict__ cache, const int* __restrict__ slot_map, int page) {
+                    T* __restrict__ q_out, int q_ld, T* __restrict__ cache, const int* __restrict__ slot_map, int page,
+                    int v_from_k, int pass_cols, float mag) {
   __shared__ float cs[PREP_MAX_HALF], sn[PREP_MAX_HALF];
   __shared__ float inv[PREP_MAX_GROUPS];               // queries' groups first, then the keys'
   const int n = blockIdx.x, lane = threadIdx.x % DA_WAVE, wave = threadIdx.x / DA_WAVE;
@@ -35,8 +40,8 @@ attn_prepare_kernel(const float* __restrict__ raw, int ld, int Hq, int Hkv, int 
     for (int i = threadIdx.x; i < half; i += PREP_THREADS) {
       double s, c;
       sincos(p * speeds[i], &s, &c);
-      cs[i] = (float)c;
-      sn[i] = (float)s;
+      cs[i] = (float)c * mag;
+      sn[i] = (float)s * mag;
     }
   }
   if (normed) {
@@ -82,21 +87,28 @@ attn_prepare_kernel(const float* __restrict__ raw, int ld, int Hq, int Hkv, int 
     else from_f32(&kbase[((long long)h * page + prow) * D + d], val);
   }
   if (slot >= 0) {
-    const float* v = row + (Hq + Hkv) * D;
+    const float* v = row + (v_from_k ? Hq : Hq + Hkv) * D;
     T* vb = kbase + (long long)Hkv * page * D;
     for (int idx = threadIdx.x; idx < Hkv * Dv; idx += PREP_THREADS) {
       const int h = idx / Dv, d = idx % Dv;
-      from_f32(&vb[((long long)h * Dv + d) * page + prow], v[idx]);
+      float val = v[idx];
+      if (v_from_k && normed) val *= inv[q_groups + (whole ? 0 : h)] * load_param(gk, gk_dtype, whole ? idx : d);
+      from_f32(&vb[((long long)h * Dv + d) * page + prow], val);
     }
   }
+  const float* extra = row + (Hq + Hkv) * D + (v_from_k ? 0 : Hkv * Dv);
+  for (int idx = threadIdx.x; idx < pass_cols; idx += PREP_THREADS) from_f32(&q_out[(size_t)n * q_ld + Hq * D + idx], extra[idx]);
 }
 
 extern "C" int da_attn_prepare(const float* raw, int ld, int Hq, int Hkv, int D, int Dv, const void* gq, int gq_dtype,
                                const void* gk, int gk_dtype, float eps, int whole, const int* positions,
                                const double* speeds, int dims, int interleaved, void* q_out, int out_dtype, int q_ld,
-                               void* cache, const int* slot_map, int page, int N, void* stream) {
-  DA_REQUIRE(N >= 0 && Hq > 0 && Hkv > 0 && D > 0 && Dv > 0 && page > 0, "attn_prepare: bad sizes");
-  DA_REQUIRE(ld >= (Hq + Hkv) * D + Hkv * Dv && q_ld >= Hq * D, "attn_prepare: row lengths too small");
+                               void* cache, const int* slot_map, int page, int N, int v_from_k, int pass_cols, float mag,
+                               void* stream) {
+  DA_REQUIRE(N >= 0 && Hq > 0 && Hkv > 0 && D > 0 && Dv > 0 && page > 0 && pass_cols >= 0, "attn_prepare: bad sizes");
+  DA_REQUIRE(!v_from_k || Dv == D, "attn_prepare: values that are the keys have the keys' size %d, not %d", D, Dv);
+  DA_REQUIRE(ld >= (Hq + Hkv) * D + (v_from_k ? 0 : Hkv * Dv) + pass_cols && q_ld >= Hq * D + pass_cols,
+             "attn_prepare: row lengths too small");
   DA_REQUIRE((gq == nullptr) == (gk == nullptr), "attn_prepare: a norm needs both gains");
   DA_REQUIRE(gq == nullptr || eps > 0.f, "attn_prepare: the norm needs a positive eps");
   DA_REQUIRE(dims >= 0 && dims <= D && dims % 2 == 0 && dims / 2 <= PREP_MAX_HALF, "attn_prepare: %d turned entries of %d", dims, D);
@@ -107,11 +119,11 @@ extern "C" int da_attn_prepare(const float* raw, int ld, int Hq, int Hkv, int D,
   if (out_dtype == DA_BF16)
     hipLaunchKernelGGL(attn_prepare_kernel<bf16_t>, dim3(N), dim3(PREP_THREADS), 0, (hipStream_t)stream, raw, ld, Hq, Hkv, D,
                        Dv, gq, gq_dtype, gk, gk_dtype, eps, whole, positions, speeds, dims, interleaved, (bf16_t*)q_out, q_ld,
-                       (bf16_t*)cache, slot_map, page);
+                       (bf16_t*)cache, slot_map, page, v_from_k, pass_cols, mag);
   else
     hipLaunchKernelGGL(attn_prepare_kernel<float>, dim3(N), dim3(PREP_THREADS), 0, (hipStream_t)stream, raw, ld, Hq, Hkv, D,
                        Dv, gq, gq_dtype, gk, gk_dtype, eps, whole, positions, speeds, dims, interleaved, (float*)q_out, q_ld,
-                       (float*)cache, slot_map, page);
+                       (float*)cache, slot_map, page, v_from_k, pass_cols, mag);
   DA_CHECK_LAUNCH("attn_prepare");
   return 0;
 }

@@ -104,7 +104,8 @@ _ARGTYPES = {
     "da_attn_window": [_VP, _I, _VP, _VP, _I, _VP, _VP, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _VP, _VP, _I, _VP, _I, _I,
                        _VP],
     "da_attn_window_takes": [_I, _I, _I],
-    "da_attn_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _I, _VP, _VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _I, _VP],
+    "da_attn_prepare": [_VP, _I, _I, _I, _I, _I, _VP, _I, _VP, _I, _F, _I, _VP, _VP, _I, _I, _VP, _I, _I, _VP, _VP, _I, _I, _I, _I, _F,
+                        _VP],
     "da_delta_rule": [_VP, _I, _I, _I, _I, _VP, _I, _VP, _I, _I, _VP, _VP, _VP, ctypes.c_long, _VP, _VP, _VP, _I, _I, _I, _I, _I,
                       _I, _I, _F, _I, _I, _VP],
     "da_delta_gate_norm": [_VP, _I, _VP, _I, _I, _VP, _I, _F, _I, _VP, _I, _I, _I, _I, _VP],
@@ -1583,19 +1584,24 @@ PREPARE_MAX_ROT = 256        # turned entries a head that ``attn_prepare`` takes
 def attn_prepare(raw: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int, v_head_dim: int,
                  q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps: float, whole: bool,
                  positions: torch.Tensor, speeds: Optional[torch.Tensor], dims: int, interleaved: bool, q_out: torch.Tensor,
-                 cache_slot: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], page: int) -> torch.Tensor:
+                 cache_slot: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], page: int,
+                 values_are_keys: bool = False, pass_cols: int = 0, magnitude: float = 1.0) -> torch.Tensor:
     """From the 32-bit rows of a q | k | v product: queries and keys normalised (``whole``: one root mean square
     over all of a token's query entries and one over all its key entries, gains of those lengths; else head by
     head with gains of ``head_dim`` entries; no gains: no norm), their first ``dims`` entries turned by the
     position (``speeds`` float64 [dims / 2]; pairs (2i, 2i + 1) when ``interleaved``, else (i, i + dims / 2)),
     the queries stored in ``q_out`` and keys and values in their cache rows ``slot_map`` (a page of the slot
-    holds Hkv * page * D keys, then Hkv * Dv * page values)."""
+    holds Hkv * page * D keys, then Hkv * Dv * page values).  ``values_are_keys``: the rows hold q | k only, and a key
+    before its turn is also the value.  ``pass_cols``: so many columns behind q | k | v go over into ``q_out`` behind the
+    queries, converted.  ``magnitude`` multiplies sine and cosine."""
     _dev(raw, q_gain, k_gain, positions, speeds, q_out, cache_slot, slot_map)
     _rows_2d(raw, "raw"); _rows_2d(q_out, "q_out")
     N = raw.shape[0]
-    q_cols, k_cols, v_cols = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_head_dim
-    _need(raw.dtype == torch.float32 and raw.shape[1] >= q_cols + k_cols + v_cols, "attn_prepare: raw must be float32 [N, q | k | v]")
-    _need(q_out.shape[0] == N and q_out.shape[1] >= q_cols, "attn_prepare: q_out must be [N, Hq * D]")
+    q_cols, k_cols, v_cols = n_heads * head_dim, n_kv_heads * head_dim, 0 if values_are_keys else n_kv_heads * v_head_dim
+    _need(not values_are_keys or v_head_dim == head_dim, "attn_prepare: values that are the keys have the keys' size")
+    _need(raw.dtype == torch.float32 and pass_cols >= 0 and raw.shape[1] >= q_cols + k_cols + v_cols + pass_cols,
+          "attn_prepare: raw must be float32 [N, q | k | v | what passes]")
+    _need(q_out.shape[0] == N and q_out.shape[1] >= q_cols + pass_cols, "attn_prepare: q_out must be [N, Hq * D + what passes]")
     _need((q_gain is None) == (k_gain is None), "attn_prepare: a norm needs both gains")
     if q_gain is not None:
         nq, nk = (q_cols, k_cols) if whole else (head_dim, head_dim)
@@ -1617,7 +1623,8 @@ def attn_prepare(raw: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: int
                                       _dt(k_gain) if k_gain is not None else 0, float(eps), int(bool(whole)), _ptr(positions),
                                       _ptr(speeds) if dims else None, int(dims), int(bool(interleaved)), _ptr(q_out),
                                       _dt(q_out), q_out.stride(0), _ptr(cache_slot),
-                                      _ptr(slot_map) if cache_slot is not None else None, int(page), N, _stream()))
+                                      _ptr(slot_map) if cache_slot is not None else None, int(page), N,
+                                      int(bool(values_are_keys)), int(pass_cols), float(magnitude), _stream()))
     return q_out
 
 

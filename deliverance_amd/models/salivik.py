@@ -6,7 +6,7 @@ latent-attention mixer ``l<i>.mix.{dq, dq.norm, uq, dkv, dkv.norm, uk, uv, sink,
 ``l<i>.mlp.{gate, up, down}``; a routed one ``l<i>.mlp.router``, ``l<i>.mlp.router.b``, ``l<i>.mlp.e<j>.{gate, up,
 down}`` and ``l<i>.mlp.shared.{gate, up, down}``.  Linear weights are stored [out, in].  Gate and up of a
 feed-forward become one matrix and the experts of a layer one stack at load time; an attention mixer's one
-product gives q | k | v | gate with the key matrix standing twice (the values are the keys before their turn).
+product gives q | k | gate (the values are the keys before their turn).
 """
 from __future__ import annotations
 
@@ -90,8 +90,8 @@ def bind_tensors(mc: ModelConfig, t: dict) -> dict:
         p, m, f = spec.weight_prefix, spec.mixer, spec.feed_forward
         d = {"pre_mixer_norm": {"weight": t[p + "norm1"]}}
         if isinstance(m, AttentionSpec):
-            # q | k | v | gate in one product; the value rows are the key matrix once more
-            d["mixer"] = {"qkv_weight": torch.cat([t[p + "mix.q"], t[p + "mix.k"], t[p + "mix.k"], t[p + "mix.g"]], dim=0),
+            # q | k | gate in one product
+            d["mixer"] = {"qkv_weight": torch.cat([t[p + "mix.q"], t[p + "mix.k"], t[p + "mix.g"]], dim=0),
                           "out_weight": t[p + "mix.o"]}
         elif isinstance(m, RetentionSpec):
             d["mixer"] = {"q_weight": t[p + "mix.q"], "k_weight": t[p + "mix.k"], "v_weight": t[p + "mix.v"],

@@ -11,10 +11,10 @@ the position (``query_temperature``), a root-mean-square norm of queries and key
 (``qk_norm``: over a token's whole projection or head by head), a cap on the scores (``score_softcap``:
 cap * tanh(score / cap)), and first keys of a sequence that a window never leaves behind (``keep_first``:
 position i sees j <= i when i - j < window or j < keep_first), values that are the keys before their rotation
-(``values_are_keys``: the caller stacks the key matrix twice into the one projection, so the product gives them), a
-term without key or value in the softmax's denominator (``sink``: exp(0), or exp of a learned number per head), and a
-logistic gate of one more projection of the input on the heads' results (``out_gate``: its rows are stacked behind
-q | k | v in the same product).
+(``values_are_keys``: the projection has no value rows; the kernel that turns the keys also keeps them unturned as
+values), a term without key or value in the softmax's denominator (``sink``: exp(0), or exp of a learned number per
+head), and a logistic gate of one more projection of the input on the heads' results (``out_gate``: its rows are stacked
+behind q | k | v in the same product).
 Reference: core/src/main/java/io/teknek/deliverance/generator/CausalSelfAttention.java:226-420
 (projections :266-291, cache write :315-336, scores/softmax/weighted sum :458-532, output
 projection :385-408); the residual add is TransformerBlock.java:176.
@@ -68,14 +68,18 @@ class CausalSelfAttention(Mixer):
         self.kv_cols = self.n_kv_heads * self.head_dim
         self.v_cols = self.n_kv_heads * self.v_head_dim
         self.o_cols = self.n_heads * self.v_head_dim
-        self.qkv_cols = self.q_cols + self.kv_cols + self.v_cols
+        self.values_are_keys = bool(getattr(spec, "values_are_keys", False))
+        self.qkv_cols = self.q_cols + self.kv_cols + (0 if self.values_are_keys else self.v_cols)
         self.out_gate = getattr(spec, "out_gate", None)
         if self.out_gate not in (None, "sigmoid"):
             raise ValueError(f"an output gate is 'sigmoid' or None, not {self.out_gate!r}")
-        if getattr(spec, "values_are_keys", False) and self.v_head_dim != self.head_dim:
+        if self.values_are_keys and self.v_head_dim != self.head_dim:
             raise ValueError(f"values that are the keys have the keys' size {self.head_dim}, not {self.v_head_dim}")
-        self.gate_off = self.qkv_cols                 # the gate's columns in the projection's rows, when there is one
-        self.proj_cols = self.qkv_cols + (self.o_cols if self.out_gate else 0)
+        self.gate_cols = self.o_cols if self.out_gate else 0
+        self.proj_cols = self.qkv_cols + self.gate_cols            # the projection's rows: q | k | v | gate
+        # Where the attention kernel finds the gate in the rows that hold its queries: behind q | k | v where the
+        # product's rows are those rows, right behind the queries where a kernel of its own makes them ready.
+        self.gate_off = self.qkv_cols
         self.scale = float(spec.scale)
         self.window = spec.window
         self.qkv_weight = to_matrix(params["qkv_weight"], dtype, device)
@@ -137,7 +141,7 @@ class CausalSelfAttention(Mixer):
         """Whether the q|k|v product may write keys and values to the cache itself (its epilogue assumes
         keys and values of one size)."""
         return (self.position is None and self.v_head_dim == self.head_dim and self.qk_norm is None
-                and self.out_gate is None)
+                and self.out_gate is None and not self.values_are_keys)
 
     normed_into = True
 
@@ -147,10 +151,20 @@ class CausalSelfAttention(Mixer):
         N = x.shape[0]
         ln = norm.fusable_params()
         rms = getattr(norm, "rms_params", lambda: None)() if ln is None else None
-        if (ln is None and rms is None) or self.qk_norm is not None or not ops.can_fuse_ln(N, x, self.qkv_weight):
+        if (ln is None and rms is None) or not ops.can_fuse_ln(N, x, self.qkv_weight):
             return False
         slot = ctx.cache.kv[call.cache]
         group = ctx.group_of(call.cache)
+        if self._prepared():
+            # the norm and the one product in one kernel, its 32-bit sums made ready by the next
+            raw = ctx.buf("qkv_raw", N, self.proj_cols, torch.float32)
+            if ln is not None:
+                ops.linear_ln(x, None, N, ln[0], ln[1], ln[2], self.qkv_weight, self.qkv_bias, raw)
+            else:
+                ops.linear_rms(x, None, N, rms[0], rms[1], rms[2], self.qkv_weight, self.qkv_bias, raw)
+            self._attend(ctx, self._prepare(ctx, raw, slot, group, call), x if into is None else into, slot, group, call,
+                         gate_off=self.q_cols)
+            return True
         if not self._epilogue_write():
             # the norm and the one product in one kernel; the turn of q and k and the cache write follow
             qkv = ctx.buf("qkv", N, self.proj_cols, ctx.dtype)
@@ -182,26 +196,42 @@ class CausalSelfAttention(Mixer):
             # the new keys and values go to the cache in the projection's epilogue
             ops.linear(h, self.qkv_weight, self.qkv_bias, qkv, kv_cache=slot, slot_map=ctx.slot_maps[group],
                        q_cols=self.q_cols)
-        elif self.qk_norm is not None:
-            # the norms act on the product's unrounded 32-bit sums; one kernel then normalises queries and keys,
-            # turns them by the position, stores the queries and writes keys and values to the cache
-            if self.out_gate is not None:
-                raise ValueError("an output gate beside a norm of queries and keys is not built")
-            raw = ctx.buf("qkv_raw", N, self.qkv_cols, torch.float32)
+        elif self._prepared():
+            # one kernel works on the product's unrounded 32-bit sums: it normalises queries and keys (if the design
+            # has that), turns them by the position, stores the queries (and the gate behind them) and writes keys and
+            # values to the cache
+            raw = ctx.buf("qkv_raw", N, self.proj_cols, torch.float32)
             ops.linear(h, self.qkv_weight, self.qkv_bias, raw)
-            rot = self.position if hasattr(self.position, "speeds") else None
-            if self.position is not None and rot is None:
-                raise ValueError("queries and keys with a norm take a rotation or no position encoding")
-            ops.attn_prepare(raw, self.n_heads, self.n_kv_heads, self.head_dim, self.v_head_dim, self.q_gain, self.k_gain,
-                             self.qk_norm.eps, self.qk_norm.whole, ctx.positions,
-                             None if rot is None else rot.speeds, 0 if rot is None else rot.dims,
-                             True if rot is None else rot.interleaved, qkv[:, :self.q_cols],
-                             slot if call.write else None, ctx.slot_maps[group] if call.write else None,
-                             ctx.cache.page_size)
+            self._attend(ctx, self._prepare(ctx, raw, slot, group, call), x, slot, group, call, gate_off=self.q_cols)
+            return
         else:
             ops.linear(h, self.qkv_weight, self.qkv_bias, qkv)
             self._turn_and_keep(ctx, qkv, slot, group, call)
         self._attend(ctx, qkv, x, slot, group, call)
+
+    def _prepared(self) -> bool:
+        """Whether queries, keys and values go through ``ops.attn_prepare`` (a norm of queries and keys, or values
+        that are the keys; a rotation or no position encoding)."""
+        if self.qk_norm is None and not self.values_are_keys:
+            return False
+        if self.position is not None and not hasattr(self.position, "speeds"):
+            raise ValueError("queries and keys with a norm, or keys that are values, take a rotation or no position encoding")
+        return True
+
+    def _prepare(self, ctx: StepContext, raw: torch.Tensor, slot: torch.Tensor, group: int, call) -> torch.Tensor:
+        """[queries | gate] in the compute dtype from the product's 32-bit rows; keys and values into the cache."""
+        rot = self.position
+        norm = self.qk_norm
+        q = ctx.buf("q_ready", raw.shape[0], self.q_cols + self.gate_cols, ctx.dtype)
+        ops.attn_prepare(raw, self.n_heads, self.n_kv_heads, self.head_dim, self.v_head_dim,
+                         None if norm is None else self.q_gain, None if norm is None else self.k_gain,
+                         0.0 if norm is None else norm.eps, True if norm is None else norm.whole, ctx.positions,
+                         None if rot is None else rot.speeds, 0 if rot is None else rot.dims,
+                         True if rot is None else rot.interleaved, q,
+                         slot if call.write else None, ctx.slot_maps[group] if call.write else None,
+                         ctx.cache.page_size, values_are_keys=self.values_are_keys, pass_cols=self.gate_cols,
+                         magnitude=1.0 if rot is None else getattr(rot, "magnitude", 1.0))
+        return q
 
     def _turn_and_keep(self, ctx: StepContext, qkv: torch.Tensor, slot: torch.Tensor, group: int, call) -> None:
         """The position encoding of q and k in place, then keys and values into the cache."""
@@ -215,21 +245,24 @@ class CausalSelfAttention(Mixer):
                                self.n_kv_heads, self.head_dim, self.v_head_dim, ctx.cache.page_size)
 
     def _attend(self, ctx: StepContext, qkv: torch.Tensor, x: torch.Tensor, slot: torch.Tensor, group: int,
-                call) -> None:
+                call, gate_off=None) -> None:
+        """``qkv``: rows that start with the queries; with a gate it lies in the same rows from ``gate_off`` on."""
         N = qkv.shape[0]
+        gate_off = self.gate_off if gate_off is None else gate_off
         o = ctx.buf("attn_out", N, self.o_cols, ctx.dtype)
         if self.extras:
-            # with a gate, q is the projection's whole rows: queries first, the gate from ``gate_off`` on
+            # with a gate, q is the whole rows: queries first, the gate from ``gate_off`` on
             ops.paged_attention_rel(ctx, qkv if self.out_gate else qkv[:, :self.q_cols], slot, group, self.n_heads, self.n_kv_heads, self.head_dim,
                                     self.v_head_dim, self.scale, self.window, self.dist_bias, self.temp_coef,
                                     self.temp_every, o, softcap=self.softcap, keep_first=self.keep_first, sink=self.sink,
-                                    gate_col=self.gate_off if self.out_gate else -1)
+                                    gate_col=gate_off if self.out_gate else -1)
         else:
             ops.paged_attention(ctx, qkv[:, :self.q_cols], slot, group, self.n_heads, self.scale, self.window, o)
         if ctx.debug_hook is not None:      # the reference's stage names (CausalSelfAttention.java:299-301,384)
             ctx.emit(call.layer, "query_projection", qkv[:, :self.q_cols])
-            ctx.emit(call.layer, "key_projection", qkv[:, self.q_cols:self.q_cols + self.kv_cols])
-            ctx.emit(call.layer, "value_projection", qkv[:, self.q_cols + self.kv_cols:self.qkv_cols])
+            if qkv.shape[1] >= self.q_cols + self.kv_cols + self.v_cols and not self._prepared():
+                ctx.emit(call.layer, "key_projection", qkv[:, self.q_cols:self.q_cols + self.kv_cols])
+                ctx.emit(call.layer, "value_projection", qkv[:, self.q_cols + self.kv_cols:self.qkv_cols])
             ctx.emit(call.layer, "attention_value", o)
             # the output projection before its bias (CausalSelfAttention.java:406), worked out once more for the hook
             ctx.emit(call.layer, "attention_output",

@@ -182,7 +182,7 @@ class MixerBench:
             W = {"mix.q": nrm(H * D, width), "mix.k": nrm(G * D, width), "mix.g": nrm(H * D, width, s=0.5), "mix.o": nrm(width, H * D)}
             spec = AttentionSpec("attention", width, H, G, D, m["scale"], qkv_bias=False, out_bias=False, window=m["mask"]["size"],
                                  position=turn, values_are_keys=True, sink="zero", out_gate="sigmoid")
-            names = lambda t: {"qkv_weight": torch.cat([t("mix.q"), t("mix.k"), t("mix.k"), t("mix.g")]), "out_weight": t("mix.o")}
+            names = lambda t: {"qkv_weight": torch.cat([t("mix.q"), t("mix.k"), t("mix.g")]), "out_weight": t("mix.o")}
             plain = lambda h: P.attention(self.W, "", m, h)
         elif kind == "retention":
             H, D, Dv = m["heads"], m["dim"], m["vdim"]
