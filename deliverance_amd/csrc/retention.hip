@@ -194,14 +194,26 @@ __global__ void retention_carry_kernel(RetArgs A, int S) {
   const float g = A.decay[e / ((long)A.Dv * A.D)];
   const int nk = (n_tok + A.chunk - 1) / A.chunk;
   float* ends = A.ends + (size_t)s * A.n_chunks * per + e;
+  // decay^chunk and decay^(the last chunk's length), each by repeated multiplication, once
+  const int last = n_tok - (nk - 1) * A.chunk;
+  float p_last = 1.f, p_full = 1.f;
+  for (int t = 0; t < A.chunk; ++t) {
+    p_full *= g;
+    p_last = t < last ? p_full : p_last;
+  }
   float cur = ends[0];
-  for (int k = 1; k < nk; ++k) {
-    const float q = ends[(size_t)k * per];
-    ends[(size_t)k * per] = cur;
-    const int len = n_tok - k * A.chunk < A.chunk ? n_tok - k * A.chunk : A.chunk;
-    float p = 1.f;
-    for (int t = 0; t < len; ++t) p *= g;
-    cur = fmaf(p, cur, q);
+  for (int k0 = 1; k0 < nk; k0 += 8) {              // eight chunks' end states asked for at once, then walked
+    float q[8];
+#pragma unroll
+    for (int i2 = 0; i2 < 8; ++i2) q[i2] = ends[(size_t)(k0 + i2 < nk ? k0 + i2 : 0) * per];
+#pragma unroll
+    for (int i2 = 0; i2 < 8; ++i2) {
+      const int k = k0 + i2;
+      if (k < nk) {
+        ends[(size_t)k * per] = cur;
+        cur = fmaf(k == nk - 1 ? p_last : p_full, cur, q[i2]);
+      }
+    }
   }
   const int slot = A.state_slots[s];
   if (A.write && slot >= 0) A.state[(size_t)slot * A.state_ld + e] = cur;
