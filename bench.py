@@ -355,7 +355,7 @@ def salivik_config(name, n_positions=1024):
            "mask": {"size": 512}, "rot": {"base": 10000.0, "dims": 16, "scaling": {"factor": 4.0, "original": 256, "fast": 32.0, "slow": 1.0}}}
     att = {"heads": H, "kv_heads": H // 4, "dim": 64, "vdim": 64, "scale": 64 ** -0.5, "mask": {"size": 512},
            "rot": {"base": 10000.0, "dims": 32}}
-    ret = {"heads": H, "dim": 64, "vdim": 64, "decay": [1.0 - 2.0 ** (-5 - i % 8) for i in range(H)], "rot": {"base": 10000.0, "dims": 64}}
+    ret = {"heads": H, "dim": 64, "vdim": 64, "decay": [1.0 - 0.3 * 2.0 ** (-(i % 8)) for i in range(H)], "rot": {"base": 10000.0, "dims": 64}}
     f, fs = (2 * E // 3) // 8 * 8, (4 * E // 3) // 8 * 8
     mlp = {"kind": "moe", "expert": {"ff": f, "limit": 7.0}, "router": {"experts": 8, "top": 2}, "shared": {"ff": fs, "limit": 7.0}}
     kinds = (("latent_attention", lat), ("attention", att), ("retention", ret))

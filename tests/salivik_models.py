@@ -55,8 +55,8 @@ def config(vocab, width, eps, layers, loop=None):
 # and 40 keys, shorter than the prompts
 CONFIG_S = config(300, 64, 1e-5,
                   [layer(ret(2, 16, 24, (0.9, 1.0), 10000.0, 16), dense(96, 2.0)),
-                   layer(lat(2, 16, 8, 24, 24, 40, 0.2, 24, 10000.0, (4.0, 64, 8.0, 1.0)), moe(4, 2, 32, 1.0, (48, 1.5))),
-                   layer(att(4, 2, 16, 0.25, 40, 10000.0, 8), moe(4, 2, 32, 1.0, (48, 1.5))),
+                   layer(lat(2, 16, 8, 24, 24, 40, 0.2, 24, 10000.0, (4.0, 64, 8.0, 1.0)), moe(4, 2, 32, 1.25, (48, 2.0))),
+                   layer(att(4, 2, 16, 0.25, 40, 10000.0, 8), moe(4, 2, 32, 1.25, (48, 2.0))),
                    layer(ret(1, 32, 16, (0.75,), 500.0, 8), None)],
                   loop=(1, 3, 3))
 
@@ -74,7 +74,7 @@ CONFIG_T = config(130, 72, 1e-6,
 CONFIG_U = config(64, 48, 1e-5,
                   [layer(lat(1, 16, 16, 16, 16, 16, 0.25, 2, 100.0, (1.0, 32, 4.0, 2.0)), moe(1, 1, 40, 3.0)),
                    layer(att(2, 2, 24, 0.2, 1, 10000.0, 0), moe(6, 2, 16, 1.0, (64, 0.4))),
-                   layer(ret(4, 8, 8, (1.0, 0.5, 0.25, 0.96875), 10000.0, 4), dense(24, 1.0))],
+                   layer(ret(4, 8, 8, (1.0, 0.5, 0.25, 0.9375), 10000.0, 4), dense(24, 1.0))],
                   loop=(0, 1, 1))
 
 

@@ -163,7 +163,7 @@ def test_the_plain_model_written_another_way():
 def test_the_engines_speeds_are_the_plain_ones():
     from deliverance_amd.config.specs import RampedSpeedsSpec
     from deliverance_amd.parts.positions import ramped_speeds
-    for dims, base, sc in ((16, 1e6, (2.0, 1024, 32.0, 1.0)), (32, 10000.0, (4.0, 256, 16.0, 1.0)), (8, 100.0, (1.0, 32, 4.0, 2.0)),
+    for dims, base, sc in ((16, 5e4, (3.0, 512, 24.0, 2.0)), (32, 10000.0, (4.0, 256, 16.0, 1.0)), (8, 100.0, (1.0, 32, 4.0, 2.0)),
                            (24, 500.0, (16.0, 32, 4.0, 0.5))):
         plain = [base ** (-2.0 * i / dims) for i in range(dims // 2)]
         got, mag = ramped_speeds(plain, dims, base, RampedSpeedsSpec(*sc))

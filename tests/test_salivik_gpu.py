@@ -41,7 +41,7 @@ def tb(a):
 
 
 # ------------------------------------------------------------------------------------------ rotation
-@pytest.mark.parametrize("scaling", [None, (4.0, 64, 8.0, 1.0), quick((2.0, 1024, 32.0, 1.0)), (1.0, 32, 4.0, 2.0), (8.0, 16, 1.0, 0.5)])
+@pytest.mark.parametrize("scaling", [None, (4.0, 64, 8.0, 1.0), quick((3.0, 512, 24.0, 2.0)), (1.0, 32, 4.0, 2.0), (8.0, 16, 1.0, 0.5)])
 @pytest.mark.parametrize("dtype", ["float32", quick("bfloat16")])
 def test_rotation_of_halves_with_ramped_speeds(dtype, scaling):
     """Entry i is paired with entry i + dims / 2; with a scaling the slow pairs turn slower and all turned pairs grow.
@@ -101,7 +101,7 @@ def test_capped_gated_feed_forward(dtype, rows, width, inner, limit):
     assert np.abs(got - want).max() <= (2e-6 if dtype == "float32" else 2e-2) * np.abs(want).max()
 
 
-@pytest.mark.parametrize("experts,top", [(12, 4), quick(5, 1), (3, 3), (1, 1), (40, 7)])
+@pytest.mark.parametrize("experts,top", [(10, 4), quick(5, 1), (3, 3), (1, 1), (40, 7)])
 def test_router_takes_the_largest_logits_and_weighs_them_among_themselves(experts, top):
     from deliverance_amd.kernels import ops
     rng = np.random.default_rng(experts)
@@ -122,8 +122,8 @@ def test_router_takes_the_largest_logits_and_weighs_them_among_themselves(expert
 
 
 @pytest.mark.parametrize("dtype", ["float32", quick("bfloat16")])
-@pytest.mark.parametrize("rows,shape", [quick(9, (4, 2, 32, 1.0, (48, 1.5))), (150, (4, 2, 32, 1.0, (48, 1.5))),
-                                        (20, (3, 3, 20, 0.7, None)), (6, (1, 1, 40, 3.0, None)), (33, (12, 4, 24, 1.0, (8, 0.4)))])
+@pytest.mark.parametrize("rows,shape", [quick(9, (4, 2, 32, 1.25, (48, 2.0))), (150, (4, 2, 32, 1.25, (48, 2.0))),
+                                        (20, (3, 3, 20, 0.7, None)), (6, (1, 1, 40, 3.0, None)), (33, (10, 3, 24, 1.25, (8, 0.4)))])
 def test_routed_feed_forward_part(dtype, rows, shape):
     """Few rows (the grouped kernels that stream an expert's weights) and many (rows gathered by expert), with and
     without a shared expert whose limit differs from the experts'."""
@@ -278,11 +278,11 @@ ATTENTIONS = [quick(MIX(att(4, 2, 16, 0.25, 40, 10000.0, 8))),       # matrix co
               quick(MIX(att(6, 3, 32, 0.2, 1, 10000.0, 0)))]        # a token sees itself only; nothing turns
 RETENTIONS = [quick(MIX(ret(2, 16, 24, (0.9, 1.0), 10000.0, 16))),
               MIX(ret(3, 20, 12, (0.0, 0.5, 0.999), 100.0, 20)),    # rows that do not fill the lanes; a decay of 0
-              quick(MIX(ret(1, 64, 40, (0.96875,), 1e6, 32))),      # columns that do not fill the last block
-              MIX(ret(2, 136, 8, (0.99951171875, 0.25), 500.0, 0))]  # nine rows a lane; nothing turns
+              quick(MIX(ret(1, 64, 40, (0.9375,), 1e6, 32))),      # columns that do not fill the last block
+              MIX(ret(2, 136, 8, (0.9990234375, 0.25), 500.0, 0))]  # nine rows a lane; nothing turns
 LATENTS = [quick(MIX(lat(2, 16, 8, 24, 24, 40, 0.2, 24, 10000.0, (4.0, 64, 8.0, 1.0)))),
            MIX(lat(3, 8, 12, 20, 18, 27, 0.3, 300, 500.0)),          # rows of 39 entries: the plain kernel
-           quick(MIX(lat(5, 32, 32, 16, 48, 160, 0.1, 33, 10000.0, (2.0, 1024, 32.0, 1.0)))),
+           quick(MIX(lat(5, 32, 32, 16, 48, 160, 0.1, 33, 10000.0, (3.0, 512, 24.0, 2.0)))),
            MIX(lat(1, 16, 16, 16, 16, 16, 0.25, 2, 100.0))]          # a window of two keys
 
 
@@ -331,7 +331,7 @@ def marked_latent(W, r):
 
 @pytest.mark.parametrize("dtype", ["float32", quick("bfloat16")])
 @pytest.mark.parametrize("kind", ["attention", "latent_attention"])
-@pytest.mark.parametrize("window,back", [quick(72, 71), (72, 72), (40, 39), quick(40, 40), (16, 15), (16, 16), (33, 32), (33, 33),
+@pytest.mark.parametrize("window,back", [quick(56, 55), (56, 56), (24, 23), quick(24, 24), (16, 15), (16, 16), (33, 32), (33, 33),
                                          (300, 250), (300, 1)])
 def test_a_key_just_inside_and_just_outside_the_window(kind, window, back, dtype):
     """The last query matches the key ``back`` tokens before it far better than any other.  With back < window the
@@ -435,7 +435,7 @@ def test_retention_in_chunks_side_by_side(dtype, chunk):
     N, S = sum(lens), len(lens)
     cols = 2 * H * D + H * Dv
     qkv = dev(bf16(rng.normal(size=(N, cols + 5)) * 0.5), DTYPES[dtype])
-    decay = dev([0.5, 0.96875, 1.0], torch.float32)
+    decay = dev([0.5, 0.9375, 1.0], torch.float32)
     q_start = np.concatenate([[0], np.cumsum(lens)])
     state0 = rng.normal(size=(S + 1, H * Dv * D + 3)).astype(np.float32)
     ctx = SimpleNamespace(q_start=dev(q_start), state_slots=dev([4, 1, -1, 0, 3]), n_seqs=S, max_query_len=max(lens),
