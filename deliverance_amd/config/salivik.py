@@ -194,7 +194,9 @@ class SalivikConfig:
                 continue
             n0 = len(r.missing)
             wm = w + "mixer."
-            ints = {k: r.get(m, k, wm) for k in _INTS[kind]}
+            # (an attention mixer's values are its keys: a missing vdim is the keys' size)
+            ints = {k: m.get("dim") if (kind == "attention" and k == "vdim" and isinstance(m, dict) and m.get("vdim") is None)
+                    else r.get(m, k, wm) for k in _INTS[kind]}
             rot = _read_rotation(r, m, wm)
             scale = window = decay = None
             if kind == "retention":
